@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the token-log-prob path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input that is already
+resident in HBM.  The headline workload is BASELINE config 2 (the Qwen3-0.6B GRPO
+ref-logprob shape: bf16 logits [8 x 512, 151936] with a padding mask); the same JSON line
+also carries the unmasked variant and the fused lm_head + log-softmax kernel at config 3.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only row|fused]
+
+Prints ONE JSON line on stdout.  Everything else goes to stderr.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+V = 151936
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_config2(dev, seed=1234):
+    """bf16 logits [8, 512, V] ~ N(0, 3^2) + one +15 spike per row; targets 50% spike / 50% uniform;
+    lengths uniform in [64, 512]."""
+    import torch
+    g = torch.Generator(device=dev).manual_seed(seed)
+    G, L = 8, 512
+    logits = torch.empty((G, L, V), device=dev, dtype=torch.bfloat16)
+    for i in range(G):   # generate per group to bound the fp32 temporary
+        logits[i] = (torch.randn((L, V), device=dev, generator=g) * 3.0).to(torch.bfloat16)
+    spike = torch.randint(0, V, (G, L), device=dev, generator=g)
+    flat = logits.view(G * L, V)
+    rows = torch.arange(G * L, device=dev)
+    flat[rows, spike.view(-1)] = (flat[rows, spike.view(-1)].float() + 15.0).to(torch.bfloat16)
+    uniform = torch.randint(0, V, (G, L), device=dev, generator=g)
+    pick = torch.rand((G, L), device=dev, generator=g) < 0.5
+    targets = torch.where(pick, spike, uniform).to(torch.int32)
+    lengths = torch.randint(64, 513, (G,), device=dev, generator=g)
+    return logits, targets, lengths, spike
+
+
+def time_steps(fn, steps, warmup):
+    """Average milliseconds per step over `steps` back-to-back launches, by HIP events recorded on
+    the stream the kernels run on (torch's current stream, which the library launches into)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return start.elapsed_time(stop) / steps, wall_ms
+
+
+def bench_row(dev, steps, warmup):
+    import torch
+    import tome_amd
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    logits, targets, lengths, spike = make_config2(dev)
+    G, L, _ = logits.shape
+    rows = G * L
+    valid = (torch.arange(L, device=dev)[None, :] < lengths[:, None]).to(torch.int32).reshape(-1).contiguous()
+    n_valid = int(valid.sum().item())
+    flat = logits.view(rows, V)
+    tg = targets.reshape(-1).contiguous()
+    lp = torch.empty(rows, dtype=torch.float32, device=dev)
+    ws_bytes = lib.tome_row_logprob_workspace(rows, V)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def step(mask):
+        _lib.check(lib.tome_row_logprob(flat.data_ptr(), 1, rows, V, V, tg.data_ptr(),
+                                        valid.data_ptr() if mask else None, 1.0, lp.data_ptr(), None, None, None,
+                                        ws.data_ptr(), ws_bytes, stream))
+
+    # correctness gate on what is being timed: spike rows must score the closed form's ballpark
+    step(True)
+    torch.cuda.synchronize()
+    got = lp.clone()
+    assert torch.isfinite(got).all() and (got <= 1e-5).all()
+    assert (got[valid == 0] == 0).all()
+
+    ms_mask, wall_mask = time_steps(lambda: step(True), steps, warmup)
+    ms_all, wall_all = time_steps(lambda: step(False), steps, warmup)
+    bytes_mask = n_valid * V * 2
+    bytes_all = rows * V * 2
+    out = {
+        "n_valid": n_valid, "rows": rows,
+        "ms_mask": ms_mask, "ms_all": ms_all, "wall_ms_mask": wall_mask,
+        "gbs_mask": bytes_mask / (ms_mask * 1e-3) / 1e9, "gbs_all": bytes_all / (ms_all * 1e-3) / 1e9,
+        "bytes_mask": bytes_mask, "bytes_all": bytes_all,
+    }
+    del logits, flat
+    torch.cuda.empty_cache()
+    return out
+
+
+def bench_fused(dev, steps, warmup):
+    import torch
+    import tome_amd
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    n, H = 4096, 1024
+    g = torch.Generator(device=dev).manual_seed(4321)
+    hidden = torch.randn((n, H), device=dev, generator=g).to(torch.bfloat16)
+    weight = (torch.randn((V, H), device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    targets = torch.randint(0, V, (n,), device=dev, generator=g).to(torch.int32)
+    lp = torch.empty(n, dtype=torch.float32, device=dev)
+    ws_bytes = lib.tome_fused_lmhead_logprob_workspace(n, H, V)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def step():
+        _lib.check(lib.tome_fused_lmhead_logprob(hidden.data_ptr(), weight.data_ptr(), n, H, V, H, H,
+                                                 targets.data_ptr(), None, 1.0, lp.data_ptr(), None, None, None,
+                                                 ws.data_ptr(), ws_bytes, stream))
+    step()
+    torch.cuda.synchronize()
+    assert torch.isfinite(lp).all() and (lp <= 1e-5).all()
+    ms, wall = time_steps(step, steps, warmup)
+    flop = 2.0 * n * H * V
+    return {"tokens": n, "H": H, "ms": ms, "wall_ms": wall, "tflops": flop / (ms * 1e-3) / 1e12, "flop": flop}
+
+
+def cpu_baseline(sample_rows=256, budget_s=12.0):
+    """NumPy fp32 restatement of local_compute_logprobs (mlx-impl/node.py:400-404) on a bounded
+    sample of the config-2 workload: `sample_rows` rows of bf16 logits, upcast included."""
+    import numpy as np
+    import oracle
+    rng = np.random.default_rng(99)
+    x = (rng.standard_normal((sample_rows, V)) * 3.0).astype(np.float32)
+    t = rng.integers(0, V, size=sample_rows).astype(np.int32)
+    x[np.arange(sample_rows), t] += 15.0
+    bits = oracle.bf16_round(x)
+    oracle.local_compute_logprobs_f32(bits[:8], t[:8], 1.0)   # warm-up
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while time.perf_counter() < t_end and len(times) < 20:
+        t0 = time.perf_counter()
+        oracle.local_compute_logprobs_f32(bits, t, 1.0)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    out = {"value": sample_rows / med, "unit": "token-logprobs/s", "cores": 1, "kind": "port",
+           "sample": f"{sample_rows} rows x {V} bf16 logits (config-2 distribution), NumPy fp32 restatement of "
+                     f"node.py:400-404, median of {len(times)} passes"}
+    # multi-core figure: the same arithmetic in scalar C with OpenMP over rows
+    try:
+        from oracle import cport
+        threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        cport.local_compute_logprobs_c(bits[:8], t[:8], 1.0)
+        ts = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            cport.local_compute_logprobs_c(bits, t, 1.0)
+            ts.append(time.perf_counter() - t0)
+        out["multicore"] = {"value": sample_rows / min(ts), "cores": threads, "kind": "port",
+                            "sample": "same rows, scalar C + OpenMP restatement (oracle/metal_logsoftmax.c)"}
+    except Exception as e:  # the C port is optional for the baseline
+        log("cpu multicore baseline skipped:", e)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", choices=["row", "fused"], default=None)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this path is measured on ONE GPU (rows are independent; more GPUs would each run "
+            "this same kernel on their own share of the tokens). --gpus must be 1.")
+        sys.exit(2)
+
+    import torch
+    import tome_amd
+    tome_amd.load_library()          # fail loudly if the HIP library was not built
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible")
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    log("device:", torch.cuda.get_device_name(dev))
+
+    row = bench_row(dev, args.steps, args.warmup) if args.only in (None, "row") else None
+    fused = bench_fused(dev, max(5, args.steps // 2), max(2, args.warmup // 2)) if args.only in (None, "fused") else None
+    cpu = None if args.no_cpu else cpu_baseline()
+
+    line = {
+        "metric": "token-logprobs/sec + % HBM/MFMA peak at V=151936, Qwen3-0.6B shape",
+        "unit": "token-logprobs/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "data": "synthetic", "dtype": "f32",
+    }
+    if row is not None:
+        line.update({
+            "value": row["n_valid"] / (row["ms_mask"] * 1e-3),
+            "ms_per_step": row["ms_mask"],
+            "config": {"workload": "config 2: row log-softmax + target gather, bf16 logits [8x512, 151936], "
+                                   "padding mask lengths~U[64,512], fp32 out",
+                       "rows": row["rows"], "valid_rows": row["n_valid"], "vocab": V, "temperature": 1.0},
+            "roofline": {"bound": "hbm", "achieved": row["gbs_mask"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": row["gbs_mask"] / HBM_PEAK_GBS, "traffic": None,
+                         "kernel": "row_logprob_kernel<bf16>", "bytes_per_launch": row["bytes_mask"]},
+            "all_rows": {"value": row["rows"] / (row["ms_all"] * 1e-3), "ms_per_step": row["ms_all"],
+                         "roofline": {"bound": "hbm", "achieved": row["gbs_all"], "peak": HBM_PEAK_GBS,
+                                      "unit": "GB/s", "frac": row["gbs_all"] / HBM_PEAK_GBS, "traffic": None,
+                                      "bytes_per_launch": row["bytes_all"]}},
+        })
+    if fused is not None:
+        f = {"value": fused["tokens"] / (fused["ms"] * 1e-3), "unit": "token-logprobs/s", "ms_per_step": fused["ms"],
+             "dtype": "bf16 x bf16 -> f32",
+             "config": {"workload": "config 3: fused lm_head + log-softmax, hidden [4096,1024] x W [151936,1024] bf16",
+                        "tokens": fused["tokens"], "hidden": fused["H"], "vocab": V},
+             "roofline": {"bound": "mfma", "achieved": fused["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
+                          "unit": "TFLOP/s", "frac": fused["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                          "kernel": "fused_lmhead_kernel", "flop_per_launch": fused["flop"]}}
+        if row is None:
+            line.update({"value": f["value"], "ms_per_step": f["ms_per_step"], "config": f["config"],
+                         "roofline": f["roofline"], "dtype": "f32"})
+        else:
+            line["fused_lmhead"] = f
+    if cpu is not None:
+        line["cpu_baseline"] = cpu
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,115 @@
+/* C ABI of libtome_logprob.so: Tome's token-log-prob path on MI355X (gfx950).
+ *
+ * Every entry point is a plain-C function over device pointers and sizes.  The
+ * caller owns every buffer (inputs, outputs, workspace); the library never
+ * allocates, frees or keeps a pointer.  Launches are asynchronous on the HIP
+ * stream passed as `stream` (a hipStream_t cast to void*; NULL = default
+ * stream) - the caller synchronises, which mirrors MLX's lazy evaluation forced
+ * by mx.eval (mlx-impl/node.py:456).  Return value: 0 on success, a negative
+ * TOME_E_* code otherwise; nothing throws across this boundary.
+ *
+ * Conventions shared by all entry points
+ *   dtype            TOME_F32 (0) or TOME_BF16 (1)
+ *   targets          int32 token ids, one per row; an id outside [0, V) yields NaN
+ *   row_valid        nullable int32 mask, one per row; rows with 0 are not read and
+ *                    their outputs are written as 0 (argmax as -1).  It replaces the
+ *                    reference's slicing by completion length (node.py:449).
+ *   temperature      > 0 and finite; the reference maps 0 to 1.0 before the call
+ *                    (`temperature or 1.0`, node.py:451) and so must the caller.
+ *   out_*            float32 per row; any of out_lse / out_entropy / out_argmax may
+ *                    be NULL.  lse and entropy are in nats of the temperature-scaled
+ *                    logits z = x / temperature.
+ */
+#ifndef TOME_LOGPROB_H
+#define TOME_LOGPROB_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TOME_ABI_VERSION 1
+
+enum { TOME_F32 = 0, TOME_BF16 = 1 };
+
+enum {
+  TOME_OK = 0,
+  TOME_E_NULL = -1,        /* a required pointer is NULL */
+  TOME_E_DTYPE = -2,       /* dtype code not supported by this entry point */
+  TOME_E_SHAPE = -3,       /* negative/zero/overflowing dimension or stride < V */
+  TOME_E_WORKSPACE = -4,   /* workspace_bytes smaller than the *_workspace() query */
+  TOME_E_TEMPERATURE = -5, /* temperature not finite or <= 0 */
+  TOME_E_ALIGN = -6,       /* pointer or stride alignment the kernel needs is not met */
+  TOME_E_HIP = -7          /* a HIP runtime call failed; see tome_last_hip_error() */
+};
+
+int tome_abi_version(void);
+const char* tome_strerror(int code);
+/* hipError_t of the last failing HIP call made by this thread inside the library (0 if none). */
+int tome_last_hip_error(void);
+
+/* ---- Row kernel: logits -> log-prob of the target id ------------------------------
+ * Replaces, for one scalar per row, both
+ *   local_compute_logprobs(logits, ids, temp)            mlx-impl/node.py:400-404
+ *   fused_log_softmax(logits, temperature)[row, token]   mlx-impl/model.py:77-89 with the
+ *                                                        host gather of node.py:571,605
+ * by one single-pass online logsumexp over each row with the target gather fused in:
+ *   out_lp[r] = x[r, t_r]/T - logsumexp_j(x[r, j]/T)
+ * `logits` is [rows, V] with `row_stride` ELEMENTS between rows (>= V).  Rows, V and
+ * strides are 64-bit: rows * V may exceed 2^31.
+ */
+size_t tome_row_logprob_workspace(int64_t rows, int64_t V);
+int tome_row_logprob(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                     const int32_t* targets, const int32_t* row_valid, float temperature,
+                     float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- Full log-softmax matrix ------------------------------------------------------
+ * fused_log_softmax(logits, temperature) as the reference returns it
+ * (mlx-impl/model.py:77-89): out[r, j] = T(x[r, j] * (1/temp)) - T(lse_r), same shape
+ * and dtype as the input, the subtraction carried out in the I/O dtype (model.py:57,60).
+ * `row_lse` is a caller-provided float32 scratch of `rows` elements.
+ */
+int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows, int64_t V,
+                          int64_t in_row_stride, int64_t out_row_stride, float temperature,
+                          float* row_lse, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- Fused lm_head + log-softmax --------------------------------------------------
+ * Replaces the pair  logits = x @ embed_tokens.weight.T  (mlx-impl/model.py:538)  +
+ * local_compute_logprobs (mlx-impl/node.py:400-404) without ever writing the
+ * [n_tokens, V] logits: bf16 MFMA over vocab tiles with an online logsumexp epilogue.
+ *   hidden  bf16 [n_tokens, H], row stride hidden_stride elements (already normalised:
+ *           the final RMSNorm of model.py:536 is the caller's)
+ *   weight  bf16 [V, H] row-major (the tied embedding matrix), row stride weight_stride
+ * Products are exact bf16 x bf16, accumulated in fp32; logits are NOT rounded to bf16.
+ * Needs H % 8 == 0 and 16-byte aligned rows.
+ */
+size_t tome_fused_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V);
+int tome_fused_lmhead_logprob(const void* hidden, const void* weight, int64_t n_tokens, int64_t H,
+                              int64_t V, int64_t hidden_stride, int64_t weight_stride,
+                              const int32_t* targets, const int32_t* row_valid, float temperature,
+                              float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- GRPO policy + reference dual pass --------------------------------------------
+ * Two lm_head weight sets over the same hidden states (policy = reference + LoRA merge,
+ * mlx-impl/node.py:102-164).  Emits per token
+ *   out_lp, out_ref_lp   log-probs of the target under each weight set
+ *   out_k3               exp(d) - d - 1 with d = ref_lp - lp   (no counterpart in the
+ *                        reference: its wire format, scheduler/proto/inference.proto:108-112,
+ *                        carries only the two log-prob lists)
+ *   out_entropy          entropy of the POLICY distribution (same remark)
+ */
+size_t tome_grpo_dual_workspace(int64_t n_tokens, int64_t H, int64_t V);
+int tome_grpo_dual(const void* hidden, const void* w_policy, const void* w_ref, int64_t n_tokens,
+                   int64_t H, int64_t V, int64_t hidden_stride, int64_t weight_stride,
+                   const int32_t* targets, const int32_t* row_valid, float temperature,
+                   float* out_lp, float* out_ref_lp, float* out_k3, float* out_entropy,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TOME_LOGPROB_H */

@@ -1,0 +1,262 @@
+"""CPU restatement of Tome's token-log-prob path.  TEST INFRASTRUCTURE ONLY.
+
+This module is the checker for the HIP kernels in ``tome_amd``; it is never on
+the product path.  Every function cites the reference lines it follows
+(paths relative to the reference repository root).
+
+Two families live here:
+
+* fp64 closed forms (``lse_rows``, ``logprob_rows``, ``entropy_rows``,
+  ``k3``, ``lmhead_logits64`` ...) - the mathematical statement of what
+  ``mlx-impl/node.py:400-404`` and ``mlx-impl/model.py:16-66`` compute,
+  evaluated on exactly-upcast inputs.  These are what parity is judged against.
+* fp32 restatements that keep the reference's own arithmetic
+  (``local_compute_logprobs_f32``, ``fused_log_softmax_f32``,
+  ``process_ref_logprobs_batched``) - used for the CPU baseline timing and
+  for the entry-point bookkeeping tests.
+
+The reference's arithmetic lives partly in MLX (``mlx>=0.30.6``,
+``pyproject.toml:17``; not vendored, not installable here): ``mx.logsumexp``,
+``mx.take_along_axis``, ``mx.argmax`` and the bf16 matmul.  Their published
+definitions are restated; what pins each function is listed below.
+
+Pinning (tests/test_oracle.py):
+  lse_rows / logprob_rows   closed forms (all-equal row -> -ln V, one spike
+                            over zeros -> -log1p((V-1)e^-c)), shift invariance,
+                            temperature identity, brute force with math.fsum on
+                            V <= 16, scipy.special.logsumexp / log_softmax and
+                            torch.float64 log_softmax as independent library
+                            routines, committed golden vectors.
+  entropy_rows              H(all-equal) = ln V, 0 <= H <= ln V, brute force,
+                            scipy.stats.entropy.
+  k3                        k3 >= 0, k3 = 0 iff lp == ref_lp, series expansion
+                            d^2/2 for small d, brute force.  NOT in the
+                            reference: pinned by closed form only.
+  argmax_rows               planted ties (lowest index wins, NumPy convention).
+                            MLX's own tie/NaN rule: parity unpinned.
+  lmhead_logits64           brute-force triple loop on tiny shapes, numpy
+                            float64 matmul.  MLX bf16 rounding of the
+                            materialised logits: parity unpinned (the fused
+                            path is specified as bf16 inputs, fp32 accumulate).
+  fused_log_softmax_f32     the reference's own check restated
+                            (tests/test_logprob_comparison.py:84-102, < 5e-3
+                            vs logits - logsumexp on bf16 [1,151936]) and the
+                            tail cases of model.py:17-20,34-36.
+  local_compute_logprobs_f32  agreement with logprob_rows within 1e-5.
+  process_ref_logprobs_batched  known-answer tests on a stub model
+                            (alignment, empty completion, temperature 0,
+                            chunking, padding id 0) and the length contract of
+                            tests/test_grpo.py:78-80.
+"""
+from __future__ import annotations
+
+import math
+from typing import Callable, Sequence
+
+import numpy as np
+
+__all__ = [
+    "bf16_round", "bf16_to_f32", "to_f64", "lse_rows", "logprob_rows", "entropy_rows",
+    "argmax_rows", "k3", "lmhead_logits64", "lmhead_stats", "full_log_softmax64",
+    "local_compute_logprobs_f32", "fused_log_softmax_f32", "process_ref_logprobs_batched",
+]
+
+
+# --------------------------------------------------------------------------
+# bf16 <-> f32 (bit patterns held as uint16; weights are bf16 in the reference,
+# mlx-impl/load_weights.py:20-22)
+# --------------------------------------------------------------------------
+def bf16_round(x: np.ndarray) -> np.ndarray:
+    """float32 -> bf16 bit pattern (uint16), round-to-nearest-even."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    rounded = u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))
+    return (rounded >> np.uint32(16)).astype(np.uint16)
+
+
+def bf16_to_f32(b: np.ndarray) -> np.ndarray:
+    """bf16 bit pattern (uint16) -> float32, exact."""
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def to_f64(x: np.ndarray) -> np.ndarray:
+    """Exact upcast.  uint16 arrays are read as bf16 bit patterns."""
+    x = np.asarray(x)
+    if x.dtype == np.uint16:
+        return bf16_to_f32(x).astype(np.float64)
+    return x.astype(np.float64)
+
+
+# --------------------------------------------------------------------------
+# fp64 closed forms
+# --------------------------------------------------------------------------
+def _scaled(x: np.ndarray, temperature: float) -> np.ndarray:
+    # node.py:401 divides by temp; model.py:27 multiplies by 1/temp.  In fp64
+    # the two agree to 1e-16 relative, far below the parity tolerance.
+    return to_f64(x) / float(temperature)
+
+
+def lse_rows(x: np.ndarray, temperature: float = 1.0) -> np.ndarray:
+    """logsumexp over the last axis of x/T, fp64 (mx.logsumexp at node.py:402)."""
+    z = _scaled(x, temperature)
+    m = z.max(axis=-1, keepdims=True)
+    return (m + np.log(np.exp(z - m).sum(axis=-1, keepdims=True)))[..., 0]
+
+
+def logprob_rows(x: np.ndarray, targets: np.ndarray, temperature: float = 1.0) -> np.ndarray:
+    """lp[r] = x[r, t_r]/T - logsumexp(x[r]/T), fp64 (node.py:400-404)."""
+    z = _scaled(x, temperature)
+    t = np.asarray(targets).astype(np.int64)
+    picked = np.take_along_axis(z, t[..., None], axis=-1)[..., 0]
+    m = z.max(axis=-1, keepdims=True)
+    lse = (m + np.log(np.exp(z - m).sum(axis=-1, keepdims=True)))[..., 0]
+    return picked - lse
+
+
+def full_log_softmax64(x: np.ndarray, temperature: float = 1.0) -> np.ndarray:
+    """out[r, j] = x[r, j]/T - logsumexp(x[r]/T): the matrix model.py:16-66 writes."""
+    z = _scaled(x, temperature)
+    m = z.max(axis=-1, keepdims=True)
+    return z - (m + np.log(np.exp(z - m).sum(axis=-1, keepdims=True)))
+
+
+def entropy_rows(x: np.ndarray, temperature: float = 1.0) -> np.ndarray:
+    """H[r] = lse - sum_j p_j z_j with z = x/T, p = softmax(z).  Not in the reference."""
+    z = _scaled(x, temperature)
+    m = z.max(axis=-1, keepdims=True)
+    e = np.exp(z - m)
+    s = e.sum(axis=-1)
+    lse = m[..., 0] + np.log(s)
+    return lse - (e * z).sum(axis=-1) / s
+
+
+def argmax_rows(x: np.ndarray) -> np.ndarray:
+    """Greedy token id, first maximum wins (int(mx.argmax(logits)), node.py:897)."""
+    return np.argmax(to_f64(x), axis=-1).astype(np.int32)
+
+
+def k3(lp: np.ndarray, ref_lp: np.ndarray) -> np.ndarray:
+    """k3 = exp(d) - d - 1, d = ref_lp - lp: per-token estimator of KL(pi || pi_ref).
+
+    Not in the reference (its wire format carries only log_probs and ref_log_probs,
+    scheduler/proto/inference.proto:108-112); closed form only.
+    """
+    d = np.asarray(ref_lp, dtype=np.float64) - np.asarray(lp, dtype=np.float64)
+    return np.expm1(d) - d
+
+
+def lmhead_logits64(hidden: np.ndarray, weight: np.ndarray) -> np.ndarray:
+    """logits = hidden @ weight.T in fp64 on exactly-upcast inputs.
+
+    weight is [V, H] row-major as in model.py:538 (x @ embed_tokens.weight.T).
+    """
+    return to_f64(hidden) @ to_f64(weight).T
+
+
+def lmhead_stats(hidden: np.ndarray, weight: np.ndarray, targets: np.ndarray,
+                 temperature: float = 1.0, row_chunk: int = 64) -> dict:
+    """Row statistics of the lm_head logits without keeping the full matrix.
+
+    Returns fp64 ``lp``, ``lse``, ``entropy`` and int32 ``argmax`` plus the two
+    largest scaled logits per row (``top1``, ``top2``; tests use the gap to
+    decide whether an argmax comparison is meaningful).
+    """
+    h = to_f64(hidden)
+    w = to_f64(weight)
+    t = np.asarray(targets).astype(np.int64)
+    n = h.shape[0]
+    out = {k: np.empty(n, dtype=np.float64) for k in ("lp", "lse", "entropy", "top1", "top2")}
+    out["argmax"] = np.empty(n, dtype=np.int32)
+    for r0 in range(0, n, row_chunk):
+        r1 = min(n, r0 + row_chunk)
+        z = (h[r0:r1] @ w.T) / float(temperature)
+        m = z.max(axis=-1, keepdims=True)
+        e = np.exp(z - m)
+        s = e.sum(axis=-1)
+        lse = m[:, 0] + np.log(s)
+        out["lse"][r0:r1] = lse
+        out["lp"][r0:r1] = np.take_along_axis(z, t[r0:r1, None], axis=-1)[:, 0] - lse
+        out["entropy"][r0:r1] = lse - (e * z).sum(axis=-1) / s
+        out["argmax"][r0:r1] = np.argmax(z, axis=-1)
+        part = np.partition(z, -2, axis=-1)[:, -2:]
+        out["top1"][r0:r1] = part[:, 1]
+        out["top2"][r0:r1] = part[:, 0]
+    return out
+
+
+# --------------------------------------------------------------------------
+# fp32 restatements that keep the reference's arithmetic
+# --------------------------------------------------------------------------
+def local_compute_logprobs_f32(logits: np.ndarray, ids: np.ndarray, temp: float) -> np.ndarray:
+    """node.py:400-404 in NumPy fp32: upcast, DIVIDE by temp, logsumexp, gather, subtract."""
+    x = (bf16_to_f32(logits) if logits.dtype == np.uint16 else logits.astype(np.float32, copy=False))
+    x = x / np.float32(temp)
+    m = x.max(axis=-1, keepdims=True)
+    log_z = m + np.log(np.exp(x - m).sum(axis=-1, keepdims=True, dtype=np.float32))
+    tok = np.take_along_axis(x, np.asarray(ids).astype(np.int64)[..., None], axis=-1)[..., 0]
+    return (tok - log_z[..., 0]).astype(np.float32)
+
+
+def fused_log_softmax_f32(logits: np.ndarray, temperature: float = 1.0) -> np.ndarray:
+    """model.py:16-66 in NumPy fp32, output in the input's dtype.
+
+    Keeps the kernel's arithmetic choices: multiply by inv_temp = 1/temp
+    (model.py:27), running max floored at -1e30 (:28), fp32 sum of exp(x*inv_temp
+    - row_max) (:43-50), lse cast to the I/O dtype T before the subtraction,
+    which is itself done in T (:57,60).  The 1024-thread reduction ORDER is not
+    reproduced here (oracle/metal_logsoftmax.c does that); fp32 sums are taken
+    pairwise by NumPy.
+    """
+    is_bf16 = logits.dtype == np.uint16
+    x = bf16_to_f32(logits) if is_bf16 else logits.astype(np.float32, copy=False)
+    inv_temp = np.float32(1.0) / np.float32(temperature)
+    z = x * inv_temp
+    row_max = np.maximum(z.max(axis=-1, keepdims=True), np.float32(-1e30))
+    s = np.exp(z - row_max).sum(axis=-1, keepdims=True, dtype=np.float32)
+    lse = (row_max + np.log(s)).astype(np.float32)
+    if is_bf16:
+        lse_t = bf16_to_f32(bf16_round(lse))
+        z_t = bf16_to_f32(bf16_round(z))
+        return bf16_round(z_t - lse_t)
+    return (z - lse).astype(np.float32)
+
+
+def process_ref_logprobs_batched(prompts: Sequence, results: Sequence, G: int,
+                                 temperature: float = 1.0, *,
+                                 reference_model: Callable[[np.ndarray], np.ndarray],
+                                 max_ref_batch_size: int = 32) -> int:
+    """node.py:391-461 with NumPy in place of MLX.
+
+    ``reference_model(full_ids uint32 [B, L]) -> logits [B, L, V]`` stands in for
+    ``self.reference_model(full_ids, cache=None)[0]`` (node.py:443).  Mutates
+    ``results[p].completions[g].ref_log_probs`` via ``extend`` (node.py:458) and
+    returns the number of completion tokens scored (node.py:454).
+    """
+    all_work = []
+    for p_idx, p in enumerate(prompts):                                   # node.py:409-414
+        p_toks = list(p.tokens)
+        for g in range(G):
+            all_work.append((p_idx, g, p_toks, list(results[p_idx].completions[g].tokens)))
+    num_toks = 0
+    for c0 in range(0, len(all_work), max_ref_batch_size):               # node.py:419-421
+        chunk = all_work[c0:c0 + max_ref_batch_size]
+        seqs = [p + c[:-1] if c else p for _, _, p, c in chunk]          # node.py:427-437
+        max_len = max(len(s) for s in seqs)
+        full_ids = np.array([s + [0] * (max_len - len(s)) for s in seqs], dtype=np.uint32)  # :439-441
+        logits = reference_model(full_ids)                               # node.py:443
+        for i, (p_idx, g, p_toks, c_toks) in enumerate(chunk):           # node.py:446-454
+            if not c_toks:
+                continue
+            lo = len(p_toks) - 1
+            c_logits = logits[i, lo:lo + len(c_toks)]
+            lps = local_compute_logprobs_f32(c_logits, np.array(c_toks, dtype=np.uint32),
+                                             temperature or 1.0)        # node.py:451
+            results[p_idx].completions[g].ref_log_probs.extend(lps.tolist())  # node.py:458
+            num_toks += len(c_toks)
+    return num_toks
+
+
+def _brute_logprob(row: Sequence[float], target: int, temperature: float = 1.0) -> float:
+    """math.fsum brute force for tiny rows; used only by the oracle's own tests."""
+    z = [float(v) / temperature for v in row]
+    m = max(z)
+    return z[target] - (m + math.log(math.fsum(math.exp(v - m) for v in z)))

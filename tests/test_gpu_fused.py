@@ -1,0 +1,142 @@
+"""GPU parity of the fused lm_head + log-softmax kernels against the fp64 oracle.
+
+Oracle = exact (fp64) product of the bf16 inputs followed by the closed-form row statistics;
+tolerance 2e-3 abs (bf16 inputs, fp32 accumulation), as BASELINE states for this path.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import tome_amd
+from conftest import V_QWEN3, bf16_bits_of
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+def _inputs(dev, n, H, V, seed, h_scale=1.0, w_scale=0.02):
+    rng = np.random.default_rng(seed)
+    h = torch.from_numpy((rng.standard_normal((n, H)) * h_scale).astype(np.float32)).to(dev).to(torch.bfloat16)
+    w = torch.from_numpy((rng.standard_normal((V, H)) * w_scale).astype(np.float32)).to(dev).to(torch.bfloat16)
+    t = rng.integers(0, V, size=n).astype(np.int32)
+    return h, w, t
+
+
+@pytest.mark.parametrize("n,H,V,T,w_scale", [
+    (1, 8, 16, 1.0, 1.0), (37, 64, 300, 1.0, 0.5), (130, 72, 1000, 0.7, 0.3), (128, 1024, 2048 + 17, 1.0, 0.05),
+    (300, 256, 5000, 1.3, 0.1), (5, 200, 256, 1.0, 0.2), (129, 128, 257, 1.0, 0.2), (64, 2560, 4096, 0.7, 0.02),
+])
+def test_fused_matches_oracle_small(dev, n, H, V, T, w_scale):
+    h, w, t = _inputs(dev, n, H, V, seed=n * 7 + V, w_scale=w_scale)
+    r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), T, want_lse=True, want_entropy=True)
+    want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(w), t, T)
+    np.testing.assert_allclose(r.lp.cpu().numpy(), want["lp"], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.lse.cpu().numpy(), want["lse"], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.entropy.cpu().numpy(), want["entropy"], atol=TOL, rtol=0)
+    assert (r.lp.cpu().numpy() <= 1e-5).all()
+
+
+def test_fused_targets_on_tile_edges(dev):
+    """Target ids at the first/last row of vocab tiles, 32-row blocks and the partial last tile."""
+    V, H = 256 * 3 + 40, 128
+    ids = [0, 1, 3, 4, 7, 8, 31, 32, 127, 128, 255, 256, 257, 511, 512, 767, 768, 769, 800, V - 1]
+    n = len(ids)
+    h, w, _ = _inputs(dev, n, H, V, seed=99, w_scale=0.3)
+    t = np.array(ids, dtype=np.int32)
+    r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 1.0)
+    want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(w), t, 1.0)
+    np.testing.assert_allclose(r.lp.cpu().numpy(), want["lp"], atol=TOL, rtol=0)
+
+
+def test_fused_qwen3_06b_shape_sampled_rows(dev):
+    """Config 3 shape (H=1024, V=151936): 192 tokens against the oracle."""
+    n, H, V = 192, 1024, V_QWEN3
+    h, w, t = _inputs(dev, n, H, V, seed=2024)
+    r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 1.0, want_lse=True, want_entropy=True)
+    want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(w), t, 1.0)
+    np.testing.assert_allclose(r.lp.cpu().numpy(), want["lp"], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.lse.cpu().numpy(), want["lse"], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.entropy.cpu().numpy(), want["entropy"], atol=TOL, rtol=0)
+
+
+def test_fused_full_config3_against_row_kernel(dev):
+    """All 4096 x 151936 of config 3: fused path vs the row kernel on fp32 logits from a library GEMM.
+
+    Size-independent cross-check (the two paths share no code besides the reduction algebra); the
+    oracle pins a sample of the same rows.
+    """
+    n, H, V = 4096, 1024, V_QWEN3
+    g = torch.Generator(device=dev).manual_seed(7)
+    h = torch.randn((n, H), device=dev, generator=g).to(torch.bfloat16)
+    w = (torch.randn((V, H), device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    t = torch.randint(0, V, (n,), device=dev, generator=g, dtype=torch.int64)
+    r = tome_amd.fused_lmhead_logprobs(h, w, t, 1.0, want_lse=True)
+    logits = h.float() @ w.float().t()
+    ref = tome_amd.token_logprobs(logits, t, 1.0, want_lse=True)
+    np.testing.assert_allclose(r.lp.cpu().numpy(), ref.lp.cpu().numpy(), atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.lse.cpu().numpy(), ref.lse.cpu().numpy(), atol=TOL, rtol=0)
+    rows = np.arange(0, n, 64)
+    want = oracle.lmhead_stats(bf16_bits_of(h[rows]), bf16_bits_of(w), t.cpu().numpy()[rows], 1.0)
+    np.testing.assert_allclose(r.lp.cpu().numpy()[rows], want["lp"], atol=TOL, rtol=0)
+
+
+def test_fused_varlen_mask_temperature(dev):
+    """Config 4 flavour: [B, L, H] hidden, lengths mask, T = 0.7."""
+    B, L, H, V = 5, 70, 320, 3000
+    rng = np.random.default_rng(17)
+    h = torch.from_numpy(rng.standard_normal((B, L, H)).astype(np.float32)).to(dev).to(torch.bfloat16)
+    w = torch.from_numpy((rng.standard_normal((V, H)) * 0.1).astype(np.float32)).to(dev).to(torch.bfloat16)
+    t = rng.integers(0, V, size=(B, L)).astype(np.int32)
+    lengths = np.array([70, 0, 13, 64, 1])
+    r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 0.7, lengths=torch.from_numpy(lengths),
+                                       want_entropy=True)
+    want = oracle.lmhead_stats(bf16_bits_of(h).reshape(B * L, H), bf16_bits_of(w), t.reshape(-1), 0.7)
+    mask = (np.arange(L)[None, :] < lengths[:, None])
+    got = r.lp.cpu().numpy()
+    assert got.shape == (B, L)
+    np.testing.assert_allclose(got[mask], want["lp"].reshape(B, L)[mask], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.entropy.cpu().numpy()[mask], want["entropy"].reshape(B, L)[mask], atol=TOL, rtol=0)
+    assert (got[~mask] == 0).all() and (r.entropy.cpu().numpy()[~mask] == 0).all()
+    none = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 0.7, lengths=torch.zeros(B, dtype=torch.int64))
+    assert (none.lp.cpu().numpy() == 0).all()
+
+
+def test_grpo_dual_matches_oracle(dev):
+    """Config 5 flavour: ref = policy + small perturbation; lp, ref_lp, k3, entropy."""
+    n, H, V = 200, 512, 6000
+    rng = np.random.default_rng(5)
+    h = torch.from_numpy(rng.standard_normal((n, H)).astype(np.float32)).to(dev).to(torch.bfloat16)
+    wp32 = (rng.standard_normal((V, H)) * 0.05).astype(np.float32)
+    wp = torch.from_numpy(wp32).to(dev).to(torch.bfloat16)
+    wr = torch.from_numpy(wp32 + (rng.standard_normal((V, H)) * 0.005).astype(np.float32)).to(dev).to(torch.bfloat16)
+    t = rng.integers(0, V, size=n).astype(np.int32)
+    valid = (rng.random(n) < 0.8).astype(np.int32)
+    r = tome_amd.grpo_dual_logprobs(h, wp, wr, torch.from_numpy(t).to(dev), 0.9, row_valid=torch.from_numpy(valid).to(dev))
+    pol = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(wp), t, 0.9)
+    ref = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(wr), t, 0.9)
+    m = valid.astype(bool)
+    np.testing.assert_allclose(r.lp.cpu().numpy()[m], pol["lp"][m], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.ref_lp.cpu().numpy()[m], ref["lp"][m], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.entropy.cpu().numpy()[m], pol["entropy"][m], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.k3.cpu().numpy()[m], oracle.k3(pol["lp"], ref["lp"])[m], atol=2 * TOL, rtol=0)
+    assert (r.k3.cpu().numpy() >= -1e-6).all()
+    for o in r:
+        assert (o.cpu().numpy()[~m] == 0).all()
+    same = tome_amd.grpo_dual_logprobs(h, wp, wp, torch.from_numpy(t).to(dev), 0.9)
+    assert np.abs(same.k3.cpu().numpy()).max() == 0.0
+    np.testing.assert_array_equal(same.lp.cpu().numpy(), same.ref_lp.cpu().numpy())
+
+
+def test_fused_rejects_bad_inputs(dev):
+    h = torch.zeros((4, 64), device=dev, dtype=torch.bfloat16)
+    w = torch.zeros((100, 64), device=dev, dtype=torch.bfloat16)
+    t = torch.zeros(4, dtype=torch.int32, device=dev)
+    with pytest.raises(TypeError):
+        tome_amd.fused_lmhead_logprobs(h.float(), w, t)
+    with pytest.raises(ValueError):
+        tome_amd.fused_lmhead_logprobs(h, w[:, :32], t)
+    with pytest.raises(ValueError):
+        tome_amd.fused_lmhead_logprobs(h, w, t, 0.0)
+    with pytest.raises(ValueError):
+        tome_amd.fused_lmhead_logprobs(h[:, :60], w[:, :60].contiguous(), t)   # H % 8 != 0

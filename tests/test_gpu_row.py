@@ -1,0 +1,169 @@
+"""GPU parity of the row kernel (tome_row_logprob through the Python mirror) against the fp64 oracle.
+
+Tolerances are BASELINE's: 1e-4 abs for fp32 logits, 2e-3 abs for bf16 inputs (the bf16 -> fp32
+upcast is exact, so the bf16 cases are also held to 1e-4); target ids and argmax bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import tome_amd
+from conftest import V_QWEN3, bf16_bits_of
+
+pytestmark = pytest.mark.gpu
+TOL_F32 = 1e-4
+TOL_BF16 = 2e-3
+
+
+def _check(logits_t, targets, T, **kw):
+    r = tome_amd.token_logprobs(logits_t, torch.from_numpy(targets).to(logits_t.device), T,
+                                want_lse=True, want_entropy=True, want_argmax=True, **kw)
+    torch.cuda.synchronize()
+    x = bf16_bits_of(logits_t) if logits_t.dtype == torch.bfloat16 else logits_t.cpu().numpy()
+    return r, x
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,V,T", [
+    (1, 16, 1.0), (3, 4096, 1.0), (5, 4097, 0.7), (7, 8191, 1.3), (64, V_QWEN3, 1.0),
+    (2, 166144, 0.5), (300, 1000, 2.0), (2500, 4104, 1.0), (1, V_QWEN3, 0.7), (17, 37, 1.0),
+])
+def test_row_matches_oracle(dev, dtype, rows, V, T):
+    rng = np.random.default_rng(rows * 1000003 + V)
+    x32 = (rng.standard_normal((rows, V)) * 2.0).astype(np.float32)
+    t = rng.integers(0, V, size=rows).astype(np.int32)
+    xt = torch.from_numpy(x32).to(dev).to(dtype)
+    r, x = _check(xt, t, T)
+    tol = TOL_F32
+    np.testing.assert_allclose(r.lp.cpu().numpy(), oracle.logprob_rows(x, t, T), atol=tol, rtol=0)
+    np.testing.assert_allclose(r.lse.cpu().numpy(), oracle.lse_rows(x, T), atol=tol, rtol=0)
+    np.testing.assert_allclose(r.entropy.cpu().numpy(), oracle.entropy_rows(x, T), atol=tol, rtol=0)
+    np.testing.assert_array_equal(r.argmax.cpu().numpy(), oracle.argmax_rows(x))
+    assert (r.lp.cpu().numpy() <= 1e-6).all()
+
+
+def test_row_strided_and_misaligned_views(dev):
+    """Row slices of a [B, L, V] tensor (node.py:449) and views that break 16-byte alignment."""
+    rng = np.random.default_rng(5)
+    big = torch.from_numpy(rng.standard_normal((4, 9, 1031)).astype(np.float32)).to(dev)
+    t = rng.integers(0, 1031, size=5).astype(np.int32)
+    sl = big[2, 3:8]                       # strided rows, contiguous V
+    r, x = _check(sl, t, 0.9)
+    np.testing.assert_allclose(r.lp.cpu().numpy(), oracle.logprob_rows(x, t, 0.9), atol=TOL_F32, rtol=0)
+    np.testing.assert_array_equal(r.argmax.cpu().numpy(), oracle.argmax_rows(x))
+    odd = big[1, :5, 1:1030]               # base pointer off by one element, V = 1029
+    t2 = rng.integers(0, 1029, size=5).astype(np.int32)
+    r, _ = _check(odd, t2, 1.0)
+    x = odd.cpu().numpy()
+    np.testing.assert_allclose(r.lp.cpu().numpy(), oracle.logprob_rows(x, t2, 1.0), atol=TOL_F32, rtol=0)
+    np.testing.assert_array_equal(r.argmax.cpu().numpy(), oracle.argmax_rows(x))
+    b16 = big.to(torch.bfloat16)[0, :, 3:1027]   # bf16, base off by 6 bytes
+    t3 = rng.integers(0, 1024, size=9).astype(np.int32)
+    r, x = _check(b16, t3, 1.0)
+    np.testing.assert_allclose(r.lp.cpu().numpy(), oracle.logprob_rows(x, t3, 1.0), atol=TOL_F32, rtol=0)
+    np.testing.assert_array_equal(r.argmax.cpu().numpy(), oracle.argmax_rows(x))
+
+
+def test_closed_forms(dev):
+    V = V_QWEN3
+    flat = torch.zeros((2, V), device=dev, dtype=torch.float32) + 3.25
+    r = tome_amd.token_logprobs(flat, torch.tensor([0, V - 1], device=dev), 1.0, want_entropy=True, want_argmax=True)
+    np.testing.assert_allclose(r.lp.cpu().numpy(), -np.log(V), atol=TOL_F32)
+    np.testing.assert_allclose(r.entropy.cpu().numpy(), np.log(V), atol=TOL_F32)
+    assert r.argmax.cpu().tolist() == [0, 0]          # all tied: lowest index
+    spike = torch.zeros((1, V), device=dev, dtype=torch.bfloat16)
+    spike[0, 777] = 15.0
+    r = tome_amd.token_logprobs(spike, torch.tensor([777], device=dev), 1.0, want_argmax=True)
+    np.testing.assert_allclose(r.lp.cpu().numpy(), -np.log1p((V - 1) * np.exp(-15.0)), atol=TOL_F32)
+    assert r.argmax.item() == 777
+
+
+def test_argmax_ties_lowest_index(dev):
+    rng = np.random.default_rng(11)
+    V = 40000
+    x = rng.standard_normal((6, V)).astype(np.float32)
+    spots = [(0, [5, 39999]), (1, [12345, 12346]), (2, [39999, 7]), (3, [8, 9, 10]), (4, [2047, 2048]), (5, [39992, 39993])]
+    for r_, idx in spots:
+        x[r_, idx] = 9.5
+    for dtype in (torch.float32, torch.bfloat16):
+        xt = torch.from_numpy(x).to(dev).to(dtype)
+        r = tome_amd.token_logprobs(xt, torch.zeros(6, dtype=torch.int32, device=dev), 1.0, want_argmax=True)
+        assert r.argmax.cpu().tolist() == [min(i) for _, i in spots]
+
+
+def test_masked_rows_and_lengths(dev):
+    rng = np.random.default_rng(3)
+    G, L, V = 4, 33, 5000
+    x = torch.from_numpy(rng.standard_normal((G, L, V)).astype(np.float32)).to(dev).to(torch.bfloat16)
+    t = rng.integers(0, V, size=(G, L)).astype(np.int32)
+    lengths = np.array([33, 1, 0, 17])
+    r = tome_amd.token_logprobs(x, torch.from_numpy(t).to(dev), 1.0, lengths=torch.from_numpy(lengths),
+                                want_lse=True, want_argmax=True)
+    want = oracle.logprob_rows(bf16_bits_of(x), t, 1.0)
+    mask = np.arange(L)[None, :] < lengths[:, None]
+    got = r.lp.cpu().numpy()
+    assert got.shape == (G, L)
+    np.testing.assert_allclose(got[mask], want[mask], atol=TOL_F32, rtol=0)
+    assert (got[~mask] == 0).all() and (r.lse.cpu().numpy()[~mask] == 0).all()
+    assert (r.argmax.cpu().numpy()[~mask] == -1).all()
+
+
+def test_shift_and_temperature_identities(dev):
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((16, 30000)) * 3).astype(np.float32)
+    t = rng.integers(0, 30000, size=16).astype(np.int32)
+    tt = torch.from_numpy(t).to(dev)
+    a = tome_amd.token_logprobs(torch.from_numpy(x).to(dev), tt, 0.7).lp
+    b = tome_amd.token_logprobs(torch.from_numpy(x + 100.0).to(dev), tt, 0.7).lp
+    c = tome_amd.token_logprobs(torch.from_numpy((x / np.float32(0.7)).astype(np.float32)).to(dev), tt, 1.0).lp
+    np.testing.assert_allclose(a.cpu().numpy(), b.cpu().numpy(), atol=1e-4)
+    np.testing.assert_allclose(a.cpu().numpy(), c.cpu().numpy(), atol=1e-4)
+
+
+def test_out_of_range_target_is_nan(dev):
+    x = torch.zeros((3, 64), device=dev)
+    r = tome_amd.token_logprobs(x, torch.tensor([-1, 64, 5], device=dev), 1.0)
+    got = r.lp.cpu().numpy()
+    assert np.isnan(got[0]) and np.isnan(got[1]) and np.isfinite(got[2])
+
+
+def test_local_compute_logprobs_dropin(dev):
+    """Same call shape as node.py:451: [Lc, V] bf16 slice, uint-like ids, temp."""
+    rng = np.random.default_rng(21)
+    logits = torch.from_numpy((rng.standard_normal((2, 40, V_QWEN3)) * 3).astype(np.float32)).to(dev).to(torch.bfloat16)
+    c_toks = rng.integers(0, V_QWEN3, size=12)
+    c_logits = logits[1, 6:18]
+    lps = tome_amd.local_compute_logprobs(c_logits, torch.tensor(c_toks, device=dev), 0.8)
+    assert lps.dtype == torch.float32 and lps.shape == (12,)
+    want = oracle.logprob_rows(bf16_bits_of(c_logits), c_toks, 0.8)
+    np.testing.assert_allclose(lps.cpu().numpy(), want, atol=TOL_BF16, rtol=0)
+    np.testing.assert_allclose(lps.cpu().numpy(), want, atol=TOL_F32, rtol=0)
+    ref32 = oracle.local_compute_logprobs_f32(bf16_bits_of(c_logits), c_toks, 0.8)
+    np.testing.assert_allclose(lps.cpu().numpy(), ref32, atol=TOL_F32, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,V,T", [(1, V_QWEN3, 1.0), (3, 4096 * 2 + 1, 0.7), (64, 4096, 1.0), (5, 8192 + 384, 2.0)])
+def test_fused_log_softmax_full_matrix(dev, dtype, rows, V, T):
+    """model.py:77-89 drop-in, incl. the kernel's tail cases (V % 4096 in {0, 1, 384})."""
+    rng = np.random.default_rng(V + rows)
+    x = torch.from_numpy(rng.standard_normal((rows, V)).astype(np.float32)).to(dev).to(dtype)
+    out = tome_amd.fused_log_softmax(x, T)
+    assert out.shape == x.shape and out.dtype == x.dtype
+    if dtype == torch.float32:
+        want = oracle.full_log_softmax64(x.cpu().numpy(), T)
+        np.testing.assert_allclose(out.cpu().numpy(), want, atol=TOL_F32, rtol=0)
+        # probabilities sum to one
+        np.testing.assert_allclose(np.exp(out.cpu().numpy().astype(np.float64)).sum(-1), 1.0, atol=1e-4)
+    else:
+        bits = bf16_bits_of(x)
+        want = oracle.fused_log_softmax_f32(bits, T)           # bf16 arithmetic of model.py:57-60
+        got = bf16_bits_of(out)
+        diff = np.abs(oracle.bf16_to_f32(got) - oracle.bf16_to_f32(want))
+        # identical except where the fp32 lse sits within rounding of a bf16 tie
+        assert (diff <= 0.0625 + 1e-6).all() and (diff == 0).mean() > 0.99
+        # the reference's own bound for this kernel (tests/test_logprob_comparison.py:102)
+        if T == 1.0:
+            exp64 = oracle.full_log_softmax64(bits, 1.0)
+            assert np.abs(oracle.bf16_to_f32(got) - exp64).max() < 0.0625 + 5e-3

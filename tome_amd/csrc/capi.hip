@@ -1,0 +1,171 @@
+// extern "C" surface of libtome_logprob.so (declared in include/tome_logprob.h): argument
+// checks on the host, then the kernel launchers.  Nothing here allocates device memory.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+
+#include "../../include/tome_logprob.h"
+
+namespace tome {
+hipError_t row_logprob_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                              const int32_t* targets, const int32_t* row_valid, float temperature,
+                              float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
+                              void* workspace, hipStream_t stream);
+int row_splits_for(int64_t rows, int64_t V, int vec);
+hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t rows, int64_t V,
+                                   int64_t in_stride, int64_t out_stride, float temperature,
+                                   const float* row_lse, hipStream_t stream);
+size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights);
+hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w1, int64_t n_tokens, int64_t H,
+                               int64_t V, int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
+                               const int32_t* row_valid, float temperature, float* out_lp, float* out_lse,
+                               float* out_entropy, int32_t* out_argmax, float* out_ref_lp, float* out_k3,
+                               void* workspace, hipStream_t stream);
+}  // namespace tome
+
+namespace {
+thread_local int g_last_hip_error = 0;
+
+int hip_result(hipError_t e) {
+  if (e == hipSuccess) return TOME_OK;
+  g_last_hip_error = (int)e;
+  return TOME_E_HIP;
+}
+
+bool bad_temperature(float t) { return !(t > 0.f) || !isfinite(t); }
+
+// rows * V elements must be addressable and the flat workgroup index must fit a 32-bit grid.
+bool bad_matrix(int64_t rows, int64_t V, int64_t stride) {
+  if (rows < 0 || V <= 0 || stride < V) return true;
+  if (V > (int64_t)0x7fffffff) return true;             // unit indices are 32-bit
+  if (rows > ((int64_t)1 << 31) / 64) return true;      // rows * splits (<= 64) must fit the grid
+  if (rows > 0 && stride > INT64_MAX / 4 / rows) return true;
+  return false;
+}
+
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+}  // namespace
+
+extern "C" {
+
+int tome_abi_version(void) { return TOME_ABI_VERSION; }
+
+int tome_last_hip_error(void) { return g_last_hip_error; }
+
+const char* tome_strerror(int code) {
+  switch (code) {
+    case TOME_OK: return "ok";
+    case TOME_E_NULL: return "a required pointer is NULL";
+    case TOME_E_DTYPE: return "unsupported dtype code";
+    case TOME_E_SHAPE: return "bad shape or stride";
+    case TOME_E_WORKSPACE: return "workspace too small";
+    case TOME_E_TEMPERATURE: return "temperature must be finite and > 0";
+    case TOME_E_ALIGN: return "pointer or stride not aligned as the kernel requires";
+    case TOME_E_HIP: return "HIP runtime error (see tome_last_hip_error)";
+    default: return "unknown error code";
+  }
+}
+
+size_t tome_row_logprob_workspace(int64_t rows, int64_t V) {
+  if (rows <= 0 || V <= 0) return 0;
+  // Worst case over the vector and the element-wise path; 16 bytes per (row, split).
+  const int s_vec = tome::row_splits_for(rows, V, 8), s_one = tome::row_splits_for(rows, V, 1);
+  const int s4 = tome::row_splits_for(rows, V, 4);
+  int s = s_vec > s_one ? s_vec : s_one;
+  if (s4 > s) s = s4;
+  return s <= 1 ? 0 : align256((size_t)rows * (size_t)s * 16);
+}
+
+int tome_row_logprob(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                     const int32_t* targets, const int32_t* row_valid, float temperature, float* out_lp,
+                     float* out_lse, float* out_entropy, int32_t* out_argmax, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+  if (dtype != TOME_F32 && dtype != TOME_BF16) return TOME_E_DTYPE;
+  if (bad_matrix(rows, V, row_stride)) return TOME_E_SHAPE;
+  if (bad_temperature(temperature)) return TOME_E_TEMPERATURE;
+  if (rows == 0) return TOME_OK;
+  if (!logits) return TOME_E_NULL;
+  if (out_lp && !targets) return TOME_E_NULL;
+  if (!out_lp && !out_lse && !out_entropy && !out_argmax) return TOME_E_NULL;
+  const size_t need = tome_row_logprob_workspace(rows, V);
+  if (need > 0 && (!workspace || workspace_bytes < need)) return TOME_E_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(logits) % (dtype == TOME_F32 ? 4 : 2) != 0) return TOME_E_ALIGN;
+  return hip_result(tome::row_logprob_launch(logits, dtype, rows, V, row_stride, targets, row_valid, temperature,
+                                             out_lp, out_lse, out_entropy, out_argmax, workspace,
+                                             static_cast<hipStream_t>(stream)));
+}
+
+int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows, int64_t V,
+                          int64_t in_row_stride, int64_t out_row_stride, float temperature, float* row_lse,
+                          void* workspace, size_t workspace_bytes, void* stream) {
+  if (dtype != TOME_F32 && dtype != TOME_BF16) return TOME_E_DTYPE;
+  if (bad_matrix(rows, V, in_row_stride) || out_row_stride < V) return TOME_E_SHAPE;
+  if (bad_temperature(temperature)) return TOME_E_TEMPERATURE;
+  if (rows == 0) return TOME_OK;
+  if (!logits || !out || !row_lse) return TOME_E_NULL;
+  const int rc = tome_row_logprob(logits, dtype, rows, V, in_row_stride, nullptr, nullptr, temperature, nullptr,
+                                  row_lse, nullptr, nullptr, workspace, workspace_bytes, stream);
+  if (rc != TOME_OK) return rc;
+  return hip_result(tome::full_log_softmax_launch(logits, out, dtype, rows, V, in_row_stride, out_row_stride,
+                                                  temperature, row_lse, static_cast<hipStream_t>(stream)));
+}
+
+static int check_fused(const void* hidden, const void* w, int64_t n_tokens, int64_t H, int64_t V,
+                       int64_t hidden_stride, int64_t weight_stride, const int32_t* targets, float temperature) {
+  if (n_tokens < 0 || H <= 0 || V <= 0 || hidden_stride < H || weight_stride < H) return TOME_E_SHAPE;
+  if (V > (int64_t)0x7fffffff || n_tokens > (int64_t)0x7fffffff || H > (int64_t)1 << 20) return TOME_E_SHAPE;
+  // The kernel addresses both matrices with 32-bit byte offsets.
+  if (n_tokens * hidden_stride * 2 >= ((int64_t)1 << 32) || V * weight_stride * 2 >= ((int64_t)1 << 32))
+    return TOME_E_SHAPE;
+  if (bad_temperature(temperature)) return TOME_E_TEMPERATURE;
+  if (n_tokens == 0) return TOME_OK;
+  if (!hidden || !w || !targets) return TOME_E_NULL;
+  if (H % 8 != 0 || hidden_stride % 8 != 0 || weight_stride % 8 != 0 ||
+      reinterpret_cast<uintptr_t>(hidden) % 16 != 0 || reinterpret_cast<uintptr_t>(w) % 16 != 0)
+    return TOME_E_ALIGN;
+  return TOME_OK;
+}
+
+size_t tome_fused_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V) {
+  if (n_tokens <= 0 || H <= 0 || V <= 0) return 0;
+  return align256(tome::fused_workspace_bytes(n_tokens, H, V, 1));
+}
+
+int tome_fused_lmhead_logprob(const void* hidden, const void* weight, int64_t n_tokens, int64_t H, int64_t V,
+                              int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
+                              const int32_t* row_valid, float temperature, float* out_lp, float* out_lse,
+                              float* out_entropy, int32_t* out_argmax, void* workspace, size_t workspace_bytes,
+                              void* stream) {
+  const int rc = check_fused(hidden, weight, n_tokens, H, V, hidden_stride, weight_stride, targets, temperature);
+  if (rc != TOME_OK || n_tokens == 0) return rc;
+  if (!out_lp) return TOME_E_NULL;
+  const size_t need = tome_fused_lmhead_logprob_workspace(n_tokens, H, V);
+  if (!workspace || workspace_bytes < need) return TOME_E_WORKSPACE;
+  return hip_result(tome::fused_lmhead_launch(hidden, weight, nullptr, n_tokens, H, V, hidden_stride, weight_stride,
+                                              targets, row_valid, temperature, out_lp, out_lse, out_entropy,
+                                              out_argmax, nullptr, nullptr, workspace,
+                                              static_cast<hipStream_t>(stream)));
+}
+
+size_t tome_grpo_dual_workspace(int64_t n_tokens, int64_t H, int64_t V) {
+  if (n_tokens <= 0 || H <= 0 || V <= 0) return 0;
+  return align256(tome::fused_workspace_bytes(n_tokens, H, V, 2));
+}
+
+int tome_grpo_dual(const void* hidden, const void* w_policy, const void* w_ref, int64_t n_tokens, int64_t H,
+                   int64_t V, int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
+                   const int32_t* row_valid, float temperature, float* out_lp, float* out_ref_lp, float* out_k3,
+                   float* out_entropy, void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = check_fused(hidden, w_policy, n_tokens, H, V, hidden_stride, weight_stride, targets, temperature);
+  if (rc != TOME_OK || n_tokens == 0) return rc;
+  if (!w_ref || !out_lp || !out_ref_lp) return TOME_E_NULL;
+  if (reinterpret_cast<uintptr_t>(w_ref) % 16 != 0) return TOME_E_ALIGN;
+  const size_t need = tome_grpo_dual_workspace(n_tokens, H, V);
+  if (!workspace || workspace_bytes < need) return TOME_E_WORKSPACE;
+  return hip_result(tome::fused_lmhead_launch(hidden, w_policy, w_ref, n_tokens, H, V, hidden_stride, weight_stride,
+                                              targets, row_valid, temperature, out_lp, nullptr, out_entropy,
+                                              nullptr, out_ref_lp, out_k3, workspace,
+                                              static_cast<hipStream_t>(stream)));
+}
+
+}  // extern "C"

@@ -1,0 +1,476 @@
+// Fused lm_head + log-softmax: hidden[n, H] x weight[V, H]^T -> per-token log-prob of the
+// target id (+ lse, entropy), with the [n, V] logits living only in MFMA accumulators.
+//
+// Replaces `logits = x @ embed_tokens.weight.T` (mlx-impl/model.py:538) followed by
+// local_compute_logprobs (mlx-impl/node.py:400-404); the reference materialises the logits in
+// bf16 and upcasts them again, here bf16 x bf16 products are accumulated in fp32 and consumed
+// in place.
+//
+// Decomposition
+//   * The GEMM is computed transposed: MFMA "A" rows are vocab entries (W is [V, H], K
+//     contiguous), MFMA "B" columns are tokens (hidden is [n, H], K contiguous).  In the
+//     32x32 accumulator layout a lane then owns ONE token (lane % 32) and 16 vocab rows per
+//     block, so the softmax row statistics are per-lane registers that persist across the
+//     whole vocab sweep; only lanes l and l^32 share a token and are merged once at the end.
+//   * A workgroup (256 lanes, 4 waves as 2 vocab x 2 token) owns a 128-token tile and a
+//     contiguous range of 256-row vocab tiles.  Per vocab tile it runs the K loop (64-wide
+//     slabs staged through padded LDS, next slab prefetched into registers), then folds the
+//     256x128 accumulator tile into the running (max, sum 2^(y-m), sum y 2^(y-m)) states.
+//   * The vocab axis is split over workgroups so that ~2 workgroups per CU are resident;
+//     each writes one partial per (token, split, vocab-wave) and fused_combine_kernel merges
+//     them deterministically.
+//   * Masked tokens are compacted first (compact_rows_kernel); token tiles are built from
+//     the compacted index list, so masked rows cost no FLOPs and no HBM traffic.
+#include "common.hpp"
+
+namespace tome {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kBV = 256;                 // vocab rows per tile
+constexpr int kBT = 128;                 // tokens per tile
+constexpr int kBK = 64;                  // K slab
+constexpr int kPitch = kBK * 2 + 16;     // LDS row pitch in bytes: 16 B pad -> conflict-free b128 reads
+constexpr int kFusedWG = 256;
+constexpr int kWaveV = 128, kWaveT = 64; // per-wave tile
+constexpr int kNBV = kWaveV / 32, kNBT = kWaveT / 32;
+constexpr int kALoads = kBV * 8 / kFusedWG;  // 16-byte chunks per lane per slab (W)
+constexpr int kBLoads = kBT * 8 / kFusedWG;  // (hidden)
+constexpr int kPartsPerSplit = kBV / kWaveV;
+
+struct FusedPartial {  // 32 bytes per (token, part)
+  float mx, s, w, tx;
+  int bi;
+  int pad[3];
+};
+
+struct FusedArgs {
+  const char* hidden;
+  const char* weight;
+  const int32_t* targets;
+  const int32_t* row_index;  // compacted valid rows, or nullptr = identity
+  const int32_t* n_valid;    // device scalar, or nullptr = n_tokens
+  FusedPartial* partials;
+  uint32_t hidden_stride_b;  // bytes
+  uint32_t weight_stride_b;
+  uint32_t hidden_bytes;     // extent of the hidden matrix (< 4 GiB, checked on the host)
+  int n_tokens;
+  int H;
+  int V;
+  int n_vtiles;
+  int n_splits;
+  int n_ttiles;
+  float scale;               // log2(e) / temperature
+};
+
+// Raw buffer descriptors: 16-byte loads addressed by a 32-bit per-lane byte offset plus a
+// uniform (scalar) offset.  A per-lane offset at or past num_bytes reads as zero, which is how
+// vocab rows past V are handled; the scalar offset is not range-checked.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const char* base, uint32_t num_bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base), 0, num_bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 ld16(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uint32_t uniform_off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, uniform_off, 0);
+}
+
+template <bool ENT>
+__global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) {
+  __shared__ __attribute__((aligned(16))) char lds[(kBV + kBT) * kPitch];
+  char* ldsA = lds;
+  char* ldsB = lds + kBV * kPitch;
+
+  // XCD-aware remap: hardware deals consecutive workgroup ids round-robin over the 8 XCDs;
+  // give each XCD a contiguous block of logical ids (= a few token tiles x all splits) so the
+  // hidden tiles it touches stay in its own L2.
+  int bid = blockIdx.x;
+  const int nwg = gridDim.x;
+  if ((nwg & 7) == 0) bid = (bid & 7) * (nwg >> 3) + (bid >> 3);
+  const int ttile = bid / a.n_splits;
+  const int split = bid % a.n_splits;
+  const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
+  const int t0 = ttile * kBT;
+  if (t0 >= n_valid) return;
+  const int vt0 = (int)((int64_t)split * a.n_vtiles / a.n_splits);
+  const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / a.n_splits);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wave_v = wave & 1, wave_t = wave >> 1;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  // ---- global -> LDS staging assignment: 8 lanes cover one 128-byte row segment ----------
+  const int ld_row = tid >> 3, ld_c = tid & 7;
+  const __amdgpu_buffer_rsrc_t rsrcB = make_rsrc(a.hidden, a.hidden_bytes);
+  uint32_t boff[kBLoads];
+#pragma unroll
+  for (int j = 0; j < kBLoads; ++j) {
+    int p = t0 + ld_row + 32 * j;
+    p = p < n_valid ? p : n_valid - 1;
+    const int tok = a.row_index ? a.row_index[p] : p;
+    boff[j] = (uint32_t)tok * a.hidden_stride_b + ld_c * 16;
+  }
+  uint32_t aoff[kALoads];
+#pragma unroll
+  for (int j = 0; j < kALoads; ++j) aoff[j] = (uint32_t)(ld_row + 32 * j) * a.weight_stride_b + ld_c * 16;
+  const int st_off = ld_row * kPitch + ld_c * 16;
+
+  // ---- per-lane token state ---------------------------------------------------------------
+  RowStat st[kNBT];
+  float tx[kNBT];
+  int tgt[kNBT];
+#pragma unroll
+  for (int bt = 0; bt < kNBT; ++bt) {
+    st[bt] = stat_identity();
+    tx[bt] = -INFINITY;
+    int p = t0 + wave_t * kWaveT + bt * 32 + l32;
+    int t = -1;
+    if (p < n_valid) t = a.targets[a.row_index ? a.row_index[p] : p];
+    tgt[bt] = (t >= 0 && t < a.V) ? t : -1;
+  }
+
+  const int nk = (a.H + kBK - 1) / kBK;
+  const char* rdA = ldsA + (wave_v * kWaveV + l32) * kPitch + lh * 16;
+  const char* rdB = ldsB + (wave_t * kWaveT + l32) * kPitch + lh * 16;
+
+  for (int vt = vt0; vt < vt1; ++vt) {
+    const int v0 = vt * kBV;
+    // Descriptor rebased to this tile: per-lane offsets stay constant and rows past V fall
+    // outside num_bytes (read as zero, then masked to -inf in the epilogue).
+    const __amdgpu_buffer_rsrc_t rsrcA =
+        make_rsrc(a.weight + (int64_t)v0 * a.weight_stride_b, (uint32_t)(a.V - v0) * a.weight_stride_b);
+
+    f32x16 acc[kNBV][kNBT];
+#pragma unroll
+    for (int i = 0; i < kNBV; ++i)
+#pragma unroll
+      for (int j = 0; j < kNBT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    u32x4 ra[kALoads], rb[kBLoads];
+    const bool in0 = ld_c * 8 < a.H;
+#pragma unroll
+    for (int j = 0; j < kALoads; ++j) ra[j] = in0 ? ld16(rsrcA, aoff[j], 0) : u32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < kBLoads; ++j) rb[j] = in0 ? ld16(rsrcB, boff[j], 0) : u32x4{0, 0, 0, 0};
+
+    for (int kt = 0; kt < nk; ++kt) {
+      __syncthreads();  // every wave has finished reading the previous slab
+#pragma unroll
+      for (int j = 0; j < kALoads; ++j) *reinterpret_cast<u32x4*>(ldsA + st_off + j * 32 * kPitch) = ra[j];
+#pragma unroll
+      for (int j = 0; j < kBLoads; ++j) *reinterpret_cast<u32x4*>(ldsB + st_off + j * 32 * kPitch) = rb[j];
+      __syncthreads();
+      if (kt + 1 < nk) {  // prefetch the next slab while this one is multiplied
+        const int koff = (kt + 1) * kBK * 2;
+        const bool in = (kt + 1) * kBK + ld_c * 8 < a.H;
+#pragma unroll
+        for (int j = 0; j < kALoads; ++j) ra[j] = in ? ld16(rsrcA, aoff[j], koff) : u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < kBLoads; ++j) rb[j] = in ? ld16(rsrcB, boff[j], koff) : u32x4{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int ks = 0; ks < kBK / 16; ++ks) {
+        bf16x8 fa[kNBV], fb[kNBT];
+#pragma unroll
+        for (int i = 0; i < kNBV; ++i)
+          fa[i] = *reinterpret_cast<const bf16x8*>(rdA + i * 32 * kPitch + ks * 32);
+#pragma unroll
+        for (int j = 0; j < kNBT; ++j)
+          fb[j] = *reinterpret_cast<const bf16x8*>(rdB + j * 32 * kPitch + ks * 32);
+#pragma unroll
+        for (int i = 0; i < kNBV; ++i)
+#pragma unroll
+          for (int j = 0; j < kNBT; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+    }
+
+    // ---- epilogue: fold this tile's logits into the per-token states ----------------------
+    // Accumulator element e of block i holds vocab row  v0 + wave_v*128 + i*32 + 8*(e/4) + 4*lh + e%4.
+    const int vbase = v0 + wave_v * kWaveV + 4 * lh;
+    if (v0 + kBV > a.V) {  // last, partial vocab tile: rows past V do not exist
+#pragma unroll
+      for (int i = 0; i < kNBV; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const bool dead = vbase + i * 32 + 8 * (e / 4) + (e % 4) >= a.V;
+#pragma unroll
+          for (int j = 0; j < kNBT; ++j) acc[i][j][e] = dead ? -INFINITY : acc[i][j][e];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < kNBT; ++j) {
+      // Target capture: rare (one tile in V/256 per token), so behind a wave-uniform test.
+      const int rel = tgt[j] - (v0 + wave_v * kWaveV);
+      const bool mine = tgt[j] >= 0 && rel >= 0 && rel < kWaveV && ((rel >> 2) & 1) == lh;
+      if (__any(mine)) {
+        const int want = mine ? ((rel >> 5) * 16 + ((rel & 31) >> 3) * 4 + (rel & 3)) : -1;
+#pragma unroll
+        for (int i = 0; i < kNBV; ++i)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) tx[j] = (want == i * 16 + e) ? acc[i][j][e] : tx[j];
+      }
+      float bm[kNBV];  // per 32-row block maximum
+#pragma unroll
+      for (int i = 0; i < kNBV; ++i) {
+        float m = acc[i][j][0];
+#pragma unroll
+        for (int e = 1; e < 16; e += 2) m = fmaxf(m, fmaxf(acc[i][j][e], e + 1 < 16 ? acc[i][j][e + 1] : acc[i][j][e]));
+        bm[i] = m;
+      }
+      float cm = st[j].mx;
+      int bi = st[j].bi;
+#pragma unroll
+      for (int i = 0; i < kNBV; ++i) {
+        const bool up = bm[i] > cm;
+        bi = up ? (v0 + wave_v * kWaveV + i * 32) : bi;  // first row of the 32-row block
+        cm = fmaxf(cm, bm[i]);
+      }
+      const float resc = fast_exp2((st[j].mx - cm) * a.scale);
+      const float m = cm * a.scale;
+      float s0 = st[j].s * resc, s1 = 0.f, w0 = ENT ? st[j].w * resc : 0.f, w1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < kNBV; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; e += 2) {
+          const float x0 = acc[i][j][e], x1 = acc[i][j][e + 1];
+          const float e0 = fast_exp2(fmaf(x0, a.scale, -m));
+          const float e1 = fast_exp2(fmaf(x1, a.scale, -m));
+          s0 += e0;
+          s1 += e1;
+          if constexpr (ENT) {
+            w0 = fmaf(fmaxf(x0, kMaxFloor) * a.scale, e0, w0);
+            w1 = fmaf(fmaxf(x1, kMaxFloor) * a.scale, e1, w1);
+          }
+        }
+      st[j].mx = cm;
+      st[j].bi = bi;
+      st[j].s = s0 + s1;
+      if constexpr (ENT) st[j].w = w0 + w1;
+    }
+  }
+
+  // ---- merge the two lane halves that share a token, write one partial per token ----------
+#pragma unroll
+  for (int j = 0; j < kNBT; ++j) {
+    stat_wave_step<5>(st[j], a.scale);
+    const float txo = wave_exchange<5>(tx[j]);
+    tx[j] = fmaxf(tx[j], txo);
+    const int p = t0 + wave_t * kWaveT + j * 32 + l32;
+    if (lh == 0 && p < n_valid) {
+      const int part = split * kPartsPerSplit + wave_v;
+      FusedPartial out;
+      out.mx = st[j].mx;
+      out.s = st[j].s;
+      out.w = st[j].w;
+      out.tx = tx[j];
+      out.bi = st[j].bi;
+      out.pad[0] = out.pad[1] = out.pad[2] = 0;
+      a.partials[(int64_t)p * (a.n_splits * kPartsPerSplit) + part] = out;
+    }
+  }
+}
+
+// ---- compaction of valid rows ----------------------------------------------------------------
+// One workgroup: row_index[0 .. n_valid) = ascending indices of rows with row_valid != 0.
+// Outputs of masked rows are zeroed here.
+struct CompactArgs {
+  const int32_t* row_valid;
+  int32_t* row_index;
+  int32_t* n_valid;
+  float* out0;
+  float* out1;
+  float* out2;
+  float* out3;
+  int32_t* out_argmax;
+  int n;
+};
+
+__global__ __launch_bounds__(1024) void compact_rows_kernel(CompactArgs a) {
+  __shared__ int wave_tot[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int per = (a.n + 1023) / 1024;
+  const int r0 = tid * per, r1 = min(a.n, r0 + per);
+  int cnt = 0;
+  for (int r = r0; r < r1; ++r) cnt += a.row_valid[r] != 0;
+  int inc = cnt;  // inclusive scan inside the wave
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int up = __shfl_up(inc, off, 64);
+    if (lane >= off) inc += up;
+  }
+  if (lane == 63) wave_tot[wave] = inc;
+  __syncthreads();
+  int base = 0;
+  for (int w = 0; w < wave; ++w) base += wave_tot[w];
+  int pos = base + inc - cnt;
+  for (int r = r0; r < r1; ++r) {
+    if (a.row_valid[r] != 0) {
+      a.row_index[pos++] = r;
+    } else {
+      if (a.out0) a.out0[r] = 0.f;
+      if (a.out1) a.out1[r] = 0.f;
+      if (a.out2) a.out2[r] = 0.f;
+      if (a.out3) a.out3[r] = 0.f;
+      if (a.out_argmax) a.out_argmax[r] = -1;
+    }
+  }
+  if (tid == 1023) *a.n_valid = base + inc;
+}
+
+// ---- combine -----------------------------------------------------------------------------------
+struct CombineArgs {
+  const FusedPartial* partials;      // policy (or the only) weight set
+  const FusedPartial* partials_ref;  // second weight set, or nullptr
+  const int32_t* row_index;
+  const int32_t* n_valid;
+  float* out_lp;
+  float* out_lse;
+  float* out_entropy;
+  float* out_ref_lp;
+  float* out_k3;
+  int n_tokens;
+  int n_parts;
+  float scale;
+};
+
+__device__ __forceinline__ void combine_one(const FusedPartial* parts, int n_parts, int lane, float scale,
+                                            RowStat& st, float& tx) {
+  st = stat_identity();
+  tx = -INFINITY;
+  for (int q = lane; q < n_parts; q += 64) {
+    const FusedPartial p = parts[q];
+    RowStat o{p.mx, p.s, p.w, p.bi};
+    stat_merge(st, o, scale);
+    tx = fmaxf(tx, p.tx);
+  }
+  stat_wave_reduce(st, scale);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) tx = fmaxf(tx, __shfl_xor(tx, off, 64));
+}
+
+__global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int p = blockIdx.x * 4 + (threadIdx.x >> 6);  // compacted position, one wave each
+  const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
+  if (p >= n_valid) return;
+  const int tok = a.row_index ? a.row_index[p] : p;
+  RowStat st;
+  float tx;
+  combine_one(a.partials + (int64_t)p * a.n_parts, a.n_parts, lane, a.scale, st, tx);
+  const float m = st.mx * a.scale;
+  const float log2s = fast_log2(st.s);
+  // tx stays -inf only when the target id was outside [0, V).
+  const float lp = tx == -INFINITY ? __builtin_nanf("") : (fmaf(tx, a.scale, -m) - log2s) * kLn2;
+  float ref_lp = 0.f;
+  if (a.partials_ref) {
+    RowStat sr;
+    float txr;
+    combine_one(a.partials_ref + (int64_t)p * a.n_parts, a.n_parts, lane, a.scale, sr, txr);
+    const float mr = sr.mx * a.scale;
+    ref_lp = txr == -INFINITY ? __builtin_nanf("") : (fmaf(txr, a.scale, -mr) - fast_log2(sr.s)) * kLn2;
+  }
+  if (lane != 0) return;
+  if (a.out_lp) a.out_lp[tok] = lp;
+  if (a.out_lse) a.out_lse[tok] = (m + log2s) * kLn2;
+  if (a.out_entropy) a.out_entropy[tok] = (m + log2s - st.w / st.s) * kLn2;
+  if (a.out_ref_lp) a.out_ref_lp[tok] = ref_lp;
+  if (a.out_k3) {
+    const float d = ref_lp - lp;
+    a.out_k3[tok] = expm1f(d) - d;
+  }
+}
+
+// ---- host side -----------------------------------------------------------------------------------
+static int fused_splits(int64_t n_tokens, int64_t V) {
+  const int64_t n_ttiles = (n_tokens + kBT - 1) / kBT;
+  const int64_t n_vtiles = (V + kBV - 1) / kBV;
+  int64_t s = (512 + n_ttiles - 1) / n_ttiles;  // ~2 resident workgroups on each of 256 CUs
+  if (s > n_vtiles) s = n_vtiles;
+  if (s < 1) s = 1;
+  return (int)s;
+}
+
+// Layout: [n_valid: 256 B][row_index: n_tokens int32, 256-aligned][partials per weight set].
+static size_t off_index() { return 256; }
+static size_t off_partials(int64_t n_tokens) { return 256 + (((size_t)n_tokens * 4 + 255) & ~(size_t)255); }
+static size_t partial_bytes(int64_t n_tokens, int64_t V) {
+  return (size_t)n_tokens * (size_t)fused_splits(n_tokens, V) * kPartsPerSplit * sizeof(FusedPartial);
+}
+
+size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights) {
+  (void)H;
+  return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, V);
+}
+
+hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w1, int64_t n_tokens, int64_t H,
+                               int64_t V, int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
+                               const int32_t* row_valid, float temperature, float* out_lp, float* out_lse,
+                               float* out_entropy, int32_t* out_argmax, float* out_ref_lp, float* out_k3,
+                               void* workspace, hipStream_t stream) {
+  char* ws = static_cast<char*>(workspace);
+  int32_t* n_valid = nullptr;
+  int32_t* row_index = nullptr;
+  if (row_valid) {
+    n_valid = reinterpret_cast<int32_t*>(ws);
+    row_index = reinterpret_cast<int32_t*>(ws + off_index());
+    CompactArgs c{row_valid, row_index, n_valid, out_lp, out_lse, out_entropy, out_ref_lp, out_argmax, (int)n_tokens};
+    hipLaunchKernelGGL(compact_rows_kernel, dim3(1), dim3(1024), 0, stream, c);
+    if (out_k3) {
+      CompactArgs c2{row_valid, row_index, n_valid, out_k3, nullptr, nullptr, nullptr, nullptr, (int)n_tokens};
+      hipLaunchKernelGGL(compact_rows_kernel, dim3(1), dim3(1024), 0, stream, c2);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  FusedArgs a;
+  a.hidden = static_cast<const char*>(hidden);
+  a.targets = targets;
+  a.row_index = row_index;
+  a.n_valid = n_valid;
+  a.hidden_stride_b = (uint32_t)(hidden_stride * 2);
+  a.weight_stride_b = (uint32_t)(weight_stride * 2);
+  a.hidden_bytes = (uint32_t)(((n_tokens - 1) * hidden_stride + H) * 2);
+  a.n_tokens = (int)n_tokens;
+  a.H = (int)H;
+  a.V = (int)V;
+  a.n_vtiles = (int)((V + kBV - 1) / kBV);
+  a.n_splits = fused_splits(n_tokens, V);
+  a.n_ttiles = (int)((n_tokens + kBT - 1) / kBT);
+  a.scale = kLog2e / temperature;
+  const dim3 grid((unsigned)(a.n_ttiles * a.n_splits)), block(kFusedWG);
+  FusedPartial* p0 = reinterpret_cast<FusedPartial*>(ws + off_partials(n_tokens));
+  FusedPartial* p1 = reinterpret_cast<FusedPartial*>(ws + off_partials(n_tokens) + partial_bytes(n_tokens, V));
+
+  a.weight = static_cast<const char*>(w0);
+  a.partials = p0;
+  if (out_entropy) hipLaunchKernelGGL(fused_lmhead_kernel<true>, grid, block, 0, stream, a);
+  else hipLaunchKernelGGL(fused_lmhead_kernel<false>, grid, block, 0, stream, a);
+  if (w1) {
+    a.weight = static_cast<const char*>(w1);
+    a.partials = p1;
+    hipLaunchKernelGGL(fused_lmhead_kernel<false>, grid, block, 0, stream, a);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+
+  CombineArgs c;
+  c.partials = p0;
+  c.partials_ref = w1 ? p1 : nullptr;
+  c.row_index = row_index;
+  c.n_valid = n_valid;
+  c.out_lp = out_lp;
+  c.out_lse = out_lse;
+  c.out_entropy = out_entropy;
+  c.out_ref_lp = out_ref_lp;
+  c.out_k3 = out_k3;
+  c.n_tokens = (int)n_tokens;
+  c.n_parts = a.n_splits * kPartsPerSplit;
+  c.scale = a.scale;
+  hipLaunchKernelGGL(fused_combine_kernel, dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, stream, c);
+  (void)out_argmax;
+  return hipGetLastError();
+}
+
+}  // namespace tome

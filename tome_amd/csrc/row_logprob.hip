@@ -1,0 +1,309 @@
+// Row kernel: logits[rows, V] -> log-prob of one target id per row (+ lse, entropy, argmax).
+//
+// Replaces local_compute_logprobs (mlx-impl/node.py:400-404) and the
+// fused_log_softmax + host gather pair (mlx-impl/model.py:16-89, node.py:571,605).  The
+// reference reads each row three times and writes a full [rows, V] matrix; here each
+// element is read from HBM once with 16-byte loads and only per-row scalars are written.
+//
+// Grid: rows * splits workgroups of 256 lanes (4 wave64).  A workgroup owns a contiguous
+// range of 16-byte load units of one row, every lane keeps an online (max, sum 2^(y-m))
+// pair over the units it reads, lanes are merged by DPP / LDS-crossbar exchanges, the four
+// waves through LDS.  splits == 1 finishes in the same launch; otherwise per-split
+// partials go to the workspace and row_combine_kernel merges them (no float atomics, so
+// results do not depend on scheduling).
+#include "common.hpp"
+
+namespace tome {
+
+constexpr int kRowWG = 256;
+constexpr int kRowWaves = kRowWG / 64;
+
+template <typename T>
+struct Elem;
+template <>
+struct Elem<float> {
+  static constexpr int kVec = 4;
+  __device__ static __forceinline__ float load1(const float* p) { return *p; }
+  __device__ static __forceinline__ void unpack(const u32x4& v, float (&x)[kVec]) {
+    x[0] = __uint_as_float(v.x);
+    x[1] = __uint_as_float(v.y);
+    x[2] = __uint_as_float(v.z);
+    x[3] = __uint_as_float(v.w);
+  }
+};
+template <>
+struct Elem<uint16_t> {  // bf16 bit patterns
+  static constexpr int kVec = 8;
+  __device__ static __forceinline__ float load1(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+  __device__ static __forceinline__ void unpack(const u32x4& v, float (&x)[kVec]) {
+    x[0] = bf16_lo(v.x);
+    x[1] = bf16_hi(v.x);
+    x[2] = bf16_lo(v.y);
+    x[3] = bf16_hi(v.y);
+    x[4] = bf16_lo(v.z);
+    x[5] = bf16_hi(v.z);
+    x[6] = bf16_lo(v.w);
+    x[7] = bf16_hi(v.w);
+  }
+};
+
+template <int N>
+__device__ __forceinline__ float max_of(const float (&x)[N]) {
+  float m = x[0];
+#pragma unroll
+  for (int i = 1; i + 1 < N; i += 2) m = fmaxf(m, fmaxf(x[i], x[i + 1]));  // v_max3_f32
+  if constexpr (N % 2 == 0) m = fmaxf(m, x[N - 1]);
+  return m;
+}
+
+// Fold N values of load unit `unit` into a lane's state.
+template <int N, bool ENT, bool AMAX>
+__device__ __forceinline__ void absorb(RowStat& st, const float (&x)[N], int unit, float scale) {
+  const float cm = max_of<N>(x);
+  const float mx_new = fmaxf(st.mx, cm);
+  if constexpr (AMAX) st.bi = (cm > st.mx) ? unit : st.bi;
+  const float resc = fast_exp2((st.mx - mx_new) * scale);
+  const float m = mx_new * scale;
+  float s = st.s * resc;
+  float w = ENT ? st.w * resc : 0.f;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const float e = fast_exp2(fmaf(x[i], scale, -m));
+    s += e;
+    if constexpr (ENT) w = fmaf(fmaxf(x[i], kMaxFloor) * scale, e, w);
+  }
+  st.mx = mx_new;
+  st.s = s;
+  if constexpr (ENT) st.w = w;
+}
+
+// Workgroup reduction of the per-lane states; the result is valid in every lane of wave 0.
+__device__ __forceinline__ RowStat block_reduce(RowStat st, float scale, RowStat* lds) {
+  stat_wave_reduce(st, scale);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) lds[wave] = st;
+  __syncthreads();
+  RowStat r = lds[0];
+#pragma unroll
+  for (int w = 1; w < kRowWaves; ++w) stat_merge(r, lds[w], scale);
+  return r;
+}
+
+struct RowPartial {  // one per (row, split) in the workspace
+  float mx, s, w;
+  int bi;
+};
+
+struct RowArgs {
+  const void* logits;
+  const int32_t* targets;
+  const int32_t* row_valid;
+  float* out_lp;
+  float* out_lse;
+  float* out_entropy;
+  int32_t* out_argmax;
+  RowPartial* partials;
+  int64_t V;
+  int64_t row_stride;
+  int splits;
+  float scale;  // log2(e) / temperature
+};
+
+// Unit index -> first element and element count.  Units below n_units are full vectors;
+// units at or above it are the single trailing elements of a row whose V % kVec != 0.
+template <typename T, bool VECTOR>
+__device__ __forceinline__ int argmax_in_unit(const T* row, int64_t V, int unit, float mx) {
+  constexpr int kVec = VECTOR ? Elem<T>::kVec : 1;
+  const int64_t n_units = V / kVec;
+  // No element above the floor was seen (all -inf / NaN row): report index 0, as a first-max scan would.
+  if (unit < 0 || unit >= n_units + (V - n_units * kVec)) return 0;
+  int64_t first = (unit < n_units) ? (int64_t)unit * kVec : n_units * kVec + (unit - n_units);
+  const int count = (unit < n_units) ? kVec : 1;
+  for (int i = 0; i < count; ++i)
+    if (Elem<T>::load1(row + first + i) == mx) return (int)(first + i);
+  return (int)first;
+}
+
+template <typename T, bool ENT, bool AMAX>
+__device__ __forceinline__ void finish_row(const RowArgs& a, const T* row, int64_t r, const RowStat& st) {
+  // Called by one lane.  lp = (y_t - m - log2 s) ln2 with the same fma that fed the sum, so
+  // the target's own term is part of s and lp <= 0 up to the rounding of the merges.
+  const float m = st.mx * a.scale;
+  const float log2s = fast_log2(st.s);
+  const int32_t t = a.targets ? a.targets[r] : -1;
+  if (a.out_lp) {
+    float lp = __builtin_nanf("");
+    if (t >= 0 && t < a.V) lp = (fmaf(Elem<T>::load1(row + t), a.scale, -m) - log2s) * kLn2;
+    a.out_lp[r] = lp;
+  }
+  if (a.out_lse) a.out_lse[r] = (m + log2s) * kLn2;
+  if constexpr (ENT) a.out_entropy[r] = (m + log2s - st.w / st.s) * kLn2;
+  if constexpr (AMAX) a.out_argmax[r] = argmax_in_unit<T, true>(row, a.V, st.bi, st.mx);
+}
+
+template <typename T, bool VECTOR, bool ENT, bool AMAX>
+__global__ __launch_bounds__(kRowWG) void row_logprob_kernel(RowArgs a) {
+  constexpr int kVec = VECTOR ? Elem<T>::kVec : 1;
+  __shared__ RowStat lds[kRowWaves];
+  const int64_t r = blockIdx.x / a.splits;
+  const int split = blockIdx.x % a.splits;
+  const int tid = threadIdx.x;
+
+  if (a.row_valid && a.row_valid[r] == 0) {  // masked row: not read, outputs zeroed
+    if (split == 0 && tid == 0) {
+      if (a.out_lp) a.out_lp[r] = 0.f;
+      if (a.out_lse) a.out_lse[r] = 0.f;
+      if (ENT) a.out_entropy[r] = 0.f;
+      if (AMAX) a.out_argmax[r] = -1;
+    }
+    return;
+  }
+
+  const T* row = static_cast<const T*>(a.logits) + r * a.row_stride;
+  const int64_t n_units = a.V / kVec;
+  const int64_t per_split = (n_units + a.splits - 1) / a.splits;
+  const int64_t u0 = per_split * split;
+  const int64_t u1 = (u0 + per_split < n_units) ? u0 + per_split : n_units;
+
+  RowStat st = stat_identity();
+  if constexpr (VECTOR) {
+    const u32x4* p = reinterpret_cast<const u32x4*>(row);
+    int64_t u = u0 + tid;
+    for (; u + 3 * kRowWG < u1; u += 4 * kRowWG) {  // four 16-byte loads in flight per lane
+      const u32x4 v0 = __builtin_nontemporal_load(p + u);
+      const u32x4 v1 = __builtin_nontemporal_load(p + u + kRowWG);
+      const u32x4 v2 = __builtin_nontemporal_load(p + u + 2 * kRowWG);
+      const u32x4 v3 = __builtin_nontemporal_load(p + u + 3 * kRowWG);
+      float x[kVec];
+      Elem<T>::unpack(v0, x);
+      absorb<kVec, ENT, AMAX>(st, x, (int)u, a.scale);
+      Elem<T>::unpack(v1, x);
+      absorb<kVec, ENT, AMAX>(st, x, (int)(u + kRowWG), a.scale);
+      Elem<T>::unpack(v2, x);
+      absorb<kVec, ENT, AMAX>(st, x, (int)(u + 2 * kRowWG), a.scale);
+      Elem<T>::unpack(v3, x);
+      absorb<kVec, ENT, AMAX>(st, x, (int)(u + 3 * kRowWG), a.scale);
+    }
+    for (; u < u1; u += kRowWG) {
+      const u32x4 v = __builtin_nontemporal_load(p + u);
+      float x[kVec];
+      Elem<T>::unpack(v, x);
+      absorb<kVec, ENT, AMAX>(st, x, (int)u, a.scale);
+    }
+    // Trailing V % kVec elements: one unit each, taken by lane 0 of the last split.
+    if (split == a.splits - 1 && tid == 0) {
+      for (int64_t e = n_units * kVec; e < a.V; ++e) {
+        float x[1] = {Elem<T>::load1(row + e)};
+        absorb<1, ENT, AMAX>(st, x, (int)(n_units + (e - n_units * kVec)), a.scale);
+      }
+    }
+  } else {
+    for (int64_t u = u0 + tid; u < u1; u += kRowWG) {
+      float x[1] = {Elem<T>::load1(row + u)};
+      absorb<1, ENT, AMAX>(st, x, (int)u, a.scale);
+    }
+  }
+
+  const RowStat tot = block_reduce(st, a.scale, lds);
+  if (tid != 0) return;
+  if (a.splits == 1) {
+    if constexpr (VECTOR) {
+      finish_row<T, ENT, AMAX>(a, row, r, tot);
+    } else {
+      // Scalar path: unit index == element index.
+      RowArgs b = a;
+      b.out_argmax = nullptr;
+      finish_row<T, ENT, false>(b, row, r, tot);
+      if constexpr (AMAX) a.out_argmax[r] = tot.bi < a.V ? tot.bi : 0;
+    }
+  } else {
+    a.partials[r * a.splits + split] = RowPartial{tot.mx, tot.s, tot.w, tot.bi};
+  }
+}
+
+// One wave per row merges the per-split partials (splits <= 64).
+template <typename T, bool VECTOR, bool ENT, bool AMAX>
+__global__ __launch_bounds__(64) void row_combine_kernel(RowArgs a) {
+  const int64_t r = blockIdx.x;
+  if (a.row_valid && a.row_valid[r] == 0) return;  // outputs already zeroed by the main kernel
+  const int lane = threadIdx.x;
+  RowStat st = stat_identity();
+  if (lane < a.splits) {
+    const RowPartial p = a.partials[r * a.splits + lane];
+    st = RowStat{p.mx, p.s, p.w, p.bi};
+  }
+  stat_wave_reduce(st, a.scale);
+  if (lane != 0) return;
+  const T* row = static_cast<const T*>(a.logits) + r * a.row_stride;
+  if constexpr (VECTOR) {
+    finish_row<T, ENT, AMAX>(a, row, r, st);
+  } else {
+    RowArgs b = a;
+    b.out_argmax = nullptr;
+    finish_row<T, ENT, false>(b, row, r, st);
+    if constexpr (AMAX) a.out_argmax[r] = st.bi < a.V ? st.bi : 0;
+  }
+}
+
+template <typename T, bool VECTOR, bool ENT, bool AMAX>
+static hipError_t launch_row(const RowArgs& a, int64_t rows, hipStream_t stream) {
+  hipLaunchKernelGGL((row_logprob_kernel<T, VECTOR, ENT, AMAX>), dim3((unsigned)(rows * a.splits)),
+                     dim3(kRowWG), 0, stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || a.splits == 1) return e;
+  hipLaunchKernelGGL((row_combine_kernel<T, VECTOR, ENT, AMAX>), dim3((unsigned)rows), dim3(64), 0,
+                     stream, a);
+  return hipGetLastError();
+}
+
+template <typename T, bool VECTOR>
+static hipError_t dispatch_flags(const RowArgs& a, int64_t rows, hipStream_t stream) {
+  const bool ent = a.out_entropy != nullptr, amax = a.out_argmax != nullptr;
+  if (ent && amax) return launch_row<T, VECTOR, true, true>(a, rows, stream);
+  if (ent) return launch_row<T, VECTOR, true, false>(a, rows, stream);
+  if (amax) return launch_row<T, VECTOR, false, true>(a, rows, stream);
+  return launch_row<T, VECTOR, false, false>(a, rows, stream);
+}
+
+// How many workgroups share a row.  Large batches use one workgroup per row; small ones
+// (decode steps, the 64-row CPU-comparison case) are split so that at least ~8 workgroups
+// per CU are in flight, as long as every split keeps a few loads per lane.
+int row_splits_for(int64_t rows, int64_t V, int vec) {
+  const int64_t units = V / vec;
+  const int64_t want_wgs = 2048;
+  int64_t s = (want_wgs + rows - 1) / rows;
+  const int64_t max_by_work = units / (2 * kRowWG);  // >= 2 loads per lane per split
+  if (s > max_by_work) s = max_by_work;
+  if (s > 64) s = 64;
+  if (s < 1) s = 1;
+  return (int)s;
+}
+
+hipError_t row_logprob_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                              const int32_t* targets, const int32_t* row_valid, float temperature,
+                              float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
+                              void* workspace, hipStream_t stream) {
+  const int esize = dtype == 0 ? 4 : 2;
+  const int vec = 16 / esize;
+  const bool vector_ok = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && (row_stride % vec == 0);
+  RowArgs a;
+  a.logits = logits;
+  a.targets = targets;
+  a.row_valid = row_valid;
+  a.out_lp = out_lp;
+  a.out_lse = out_lse;
+  a.out_entropy = out_entropy;
+  a.out_argmax = out_argmax;
+  a.partials = static_cast<RowPartial*>(workspace);
+  a.V = V;
+  a.row_stride = row_stride;
+  a.splits = row_splits_for(rows, V, vector_ok ? vec : 1);
+  a.scale = kLog2e / temperature;
+  if (dtype == 0) {
+    return vector_ok ? dispatch_flags<float, true>(a, rows, stream) : dispatch_flags<float, false>(a, rows, stream);
+  }
+  return vector_ok ? dispatch_flags<uint16_t, true>(a, rows, stream)
+                   : dispatch_flags<uint16_t, false>(a, rows, stream);
+}
+
+}  // namespace tome

@@ -1,0 +1,267 @@
+"""Token-log-prob operators on torch (ROCm) tensors, backed by libtome_logprob.so.
+
+The first two functions keep the reference's names, argument order and meaning:
+
+* ``fused_log_softmax(logits, temperature=1.0)``     mlx-impl/model.py:77-89
+* ``local_compute_logprobs(logits, ids, temp)``      mlx-impl/node.py:400-404
+
+The others are the additive, fused forms of the same path: one scalar per row
+instead of a [rows, V] matrix (``token_logprobs``), the lm_head matmul of
+mlx-impl/model.py:538 folded in (``fused_lmhead_logprobs``), and the GRPO
+policy + reference pair with k3 KL and entropy (``grpo_dual_logprobs``).
+
+Launches are asynchronous on the current torch stream, like MLX's lazy graph
+(forced by ``mx.eval`` at node.py:456); reading a result on the host synchronises.
+"""
+from __future__ import annotations
+
+from typing import NamedTuple, Optional
+
+import torch
+
+from . import _lib
+from ._lib import TOME_BF16, TOME_F32
+
+
+class TokenLogprobs(NamedTuple):
+    lp: torch.Tensor                    # float32, log-prob of the target id
+    lse: Optional[torch.Tensor]         # float32, logsumexp of x / temperature
+    entropy: Optional[torch.Tensor]     # float32, entropy of softmax(x / temperature), nats
+    argmax: Optional[torch.Tensor]      # int32, first maximum of the row
+
+
+class DualLogprobs(NamedTuple):
+    lp: torch.Tensor        # policy log-prob of the target id
+    ref_lp: torch.Tensor    # reference-model log-prob of the target id
+    k3: torch.Tensor        # exp(ref_lp - lp) - (ref_lp - lp) - 1
+    entropy: torch.Tensor   # entropy of the policy distribution
+
+
+def _require_gpu(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("tome_amd operators run on a ROCm GPU only (there is no CPU fallback); "
+                               f"got a tensor on {t.device}")
+        if t.device != dev:
+            raise ValueError("all tensors must be on the same device")
+    return dev
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return TOME_F32
+    if t.dtype == torch.bfloat16:
+        return TOME_BF16
+    raise TypeError(f"logits must be float32 or bfloat16, got {t.dtype}")
+
+
+def _check_temperature(temperature: float) -> float:
+    temperature = float(temperature)
+    if not (temperature > 0.0) or temperature == float("inf"):
+        # the reference maps 0 to 1.0 at its call sites (`temperature or 1.0`, node.py:451)
+        raise ValueError(f"temperature must be finite and > 0, got {temperature}")
+    return temperature
+
+
+def _rows_view(x: torch.Tensor) -> torch.Tensor:
+    """[..., V] -> [rows, V] with unit stride along V, copying only when no such view exists."""
+    if x.dim() == 0:
+        raise ValueError("expected a tensor with a vocabulary axis")
+    V = x.shape[-1]
+    if x.dim() == 1:
+        x = x.unsqueeze(0)
+    if x.stride(-1) != 1 and V > 1:
+        x = x.contiguous()
+    if x.dim() == 2:
+        return x
+    try:
+        return x.view(-1, V)
+    except RuntimeError:
+        return x.reshape(-1, V)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _as_i32(t, n: int, dev: torch.device, what: str) -> torch.Tensor:
+    t = torch.as_tensor(t, device=dev) if not isinstance(t, torch.Tensor) else t
+    if t.device != dev:
+        raise ValueError(f"{what} must be on {dev}")
+    if t.numel() != n:
+        raise ValueError(f"{what} has {t.numel()} entries, expected {n}")
+    if t.dtype.is_floating_point or t.dtype == torch.bool:
+        raise TypeError(f"{what} must be an integer tensor")
+    return t.reshape(-1).to(torch.int32).contiguous()
+
+
+def _row_valid(lead_shape, n_rows: int, lengths, row_valid, dev) -> Optional[torch.Tensor]:
+    """Row mask from either an explicit mask or per-sequence lengths over a [B, L] leading shape."""
+    if lengths is not None and row_valid is not None:
+        raise ValueError("pass lengths or row_valid, not both")
+    if row_valid is not None:
+        rv = row_valid if isinstance(row_valid, torch.Tensor) else torch.as_tensor(row_valid, device=dev)
+        if rv.numel() != n_rows:
+            raise ValueError(f"row_valid has {rv.numel()} entries, expected {n_rows}")
+        return rv.reshape(-1).to(device=dev, dtype=torch.int32).contiguous()
+    if lengths is None:
+        return None
+    if len(lead_shape) != 2:
+        raise ValueError("lengths needs inputs shaped [batch, seq, ...]")
+    B, L = lead_shape
+    ln = lengths if isinstance(lengths, torch.Tensor) else torch.as_tensor(lengths)
+    if ln.numel() != B:
+        raise ValueError(f"lengths has {ln.numel()} entries, expected {B}")
+    ln = ln.to(device=dev, dtype=torch.int64).reshape(B, 1)
+    return (torch.arange(L, device=dev).reshape(1, L) < ln).to(torch.int32).reshape(-1).contiguous()
+
+
+def _workspace(nbytes: int, dev: torch.device) -> Optional[torch.Tensor]:
+    return torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes > 0 else None
+
+
+def token_logprobs(logits: torch.Tensor, targets, temperature: float = 1.0, lengths=None, *,
+                   row_valid=None, want_lse: bool = False, want_entropy: bool = False,
+                   want_argmax: bool = False) -> TokenLogprobs:
+    """Log-prob of ``targets`` under softmax(logits / temperature), one scalar per row.
+
+    ``logits`` is [..., V] float32 or bfloat16; ``targets`` has the leading shape.
+    Rows masked out by ``lengths`` (per sequence, for [B, L, V] inputs) or
+    ``row_valid`` are not read; their outputs are 0 (argmax -1).  Outputs are float32
+    with the leading shape.
+    """
+    lib = _lib.load_library()
+    dev = _require_gpu(logits)
+    temperature = _check_temperature(temperature)
+    dtype = _dtype_code(logits)
+    lead = tuple(logits.shape[:-1])
+    x = _rows_view(logits)
+    rows, V = x.shape
+    tg = _as_i32(targets, rows, dev, "targets")
+    rv = _row_valid(lead, rows, lengths, row_valid, dev)
+    with torch.cuda.device(dev):
+        lp = torch.empty(rows, dtype=torch.float32, device=dev)
+        lse = torch.empty(rows, dtype=torch.float32, device=dev) if want_lse else None
+        ent = torch.empty(rows, dtype=torch.float32, device=dev) if want_entropy else None
+        amax = torch.empty(rows, dtype=torch.int32, device=dev) if want_argmax else None
+        ws_bytes = lib.tome_row_logprob_workspace(rows, V)
+        ws = _workspace(ws_bytes, dev)
+        _lib.check(lib.tome_row_logprob(x.data_ptr(), dtype, rows, V, x.stride(0) if rows > 1 else V,
+                                        tg.data_ptr(), _ptr(rv), temperature, lp.data_ptr(), _ptr(lse),
+                                        _ptr(ent), _ptr(amax), _ptr(ws), ws_bytes, _stream(dev)))
+
+    def _shaped(t):
+        return None if t is None else t.reshape(lead)
+    return TokenLogprobs(_shaped(lp), _shaped(lse), _shaped(ent), _shaped(amax))
+
+
+def local_compute_logprobs(logits: torch.Tensor, ids: torch.Tensor, temp: float) -> torch.Tensor:
+    """Drop-in for the closure at mlx-impl/node.py:400-404.
+
+    ``logits`` [Lc, V] (bf16 or f32), ``ids`` [Lc] token ids, ``temp`` > 0.  Returns
+    float32 [Lc]: ``logits[ids]/temp - logsumexp(logits/temp)`` computed in fp32 in one
+    pass over the row.
+    """
+    return token_logprobs(logits, ids, temp).lp
+
+
+def fused_log_softmax(logits: torch.Tensor, temperature: float = 1.0) -> torch.Tensor:
+    """Drop-in for mlx-impl/model.py:77-89: full log-softmax with temperature, same shape and dtype."""
+    lib = _lib.load_library()
+    dev = _require_gpu(logits)
+    temperature = _check_temperature(temperature)
+    dtype = _dtype_code(logits)
+    x = _rows_view(logits)
+    rows, V = x.shape
+    with torch.cuda.device(dev):
+        out = torch.empty((rows, V), dtype=logits.dtype, device=dev)
+        row_lse = torch.empty(rows, dtype=torch.float32, device=dev)
+        ws_bytes = lib.tome_row_logprob_workspace(rows, V)
+        ws = _workspace(ws_bytes, dev)
+        _lib.check(lib.tome_full_log_softmax(x.data_ptr(), out.data_ptr(), dtype, rows, V,
+                                             x.stride(0) if rows > 1 else V, V, temperature,
+                                             row_lse.data_ptr(), _ptr(ws), ws_bytes, _stream(dev)))
+    return out.reshape(logits.shape)
+
+
+def _check_fused_inputs(hidden: torch.Tensor, *weights: torch.Tensor):
+    dev = _require_gpu(hidden, *weights)
+    if hidden.dtype != torch.bfloat16 or any(w.dtype != torch.bfloat16 for w in weights):
+        raise TypeError("hidden and lm_head weights must be bfloat16 "
+                        "(the reference loads bf16 weights, mlx-impl/load_weights.py:20-22)")
+    H = hidden.shape[-1]
+    for w in weights:
+        if w.dim() != 2 or w.shape[1] != H:
+            raise ValueError(f"weight must be [V, {H}] (rows = vocabulary, as embed_tokens.weight), got {tuple(w.shape)}")
+        if w.shape != weights[0].shape:
+            raise ValueError("policy and reference weights must have the same shape")
+    lead = tuple(hidden.shape[:-1])
+    h2 = _rows_view(hidden)
+    ws_ = [w if w.stride(1) == 1 else w.contiguous() for w in weights]
+    return dev, lead, h2, ws_
+
+
+def fused_lmhead_logprobs(hidden: torch.Tensor, weight: torch.Tensor, targets, temperature: float = 1.0,
+                          lengths=None, *, row_valid=None, want_lse: bool = False,
+                          want_entropy: bool = False) -> TokenLogprobs:
+    """Log-probs of ``targets`` under softmax((hidden @ weight.T) / temperature) without the logits.
+
+    ``hidden`` [..., H] bf16 (already through the final norm, mlx-impl/model.py:536),
+    ``weight`` [V, H] bf16 (the tied embedding matrix, model.py:538).  bf16 products are
+    accumulated in fp32; unlike the reference the logits are not rounded to bf16.
+    """
+    lib = _lib.load_library()
+    dev, lead, h2, (w,) = _check_fused_inputs(hidden, weight)
+    temperature = _check_temperature(temperature)
+    n, H = h2.shape
+    V = w.shape[0]
+    tg = _as_i32(targets, n, dev, "targets")
+    rv = _row_valid(lead, n, lengths, row_valid, dev)
+    with torch.cuda.device(dev):
+        lp = torch.empty(n, dtype=torch.float32, device=dev)
+        lse = torch.empty(n, dtype=torch.float32, device=dev) if want_lse else None
+        ent = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
+        ws_bytes = lib.tome_fused_lmhead_logprob_workspace(n, H, V)
+        ws = _workspace(ws_bytes, dev)
+        _lib.check(lib.tome_fused_lmhead_logprob(h2.data_ptr(), w.data_ptr(), n, H, V,
+                                                 h2.stride(0) if n > 1 else H, w.stride(0),
+                                                 tg.data_ptr(), _ptr(rv), temperature, lp.data_ptr(), _ptr(lse),
+                                                 _ptr(ent), None, _ptr(ws), ws_bytes, _stream(dev)))
+
+    def _shaped(t):
+        return None if t is None else t.reshape(lead)
+    return TokenLogprobs(_shaped(lp), _shaped(lse), _shaped(ent), None)
+
+
+def grpo_dual_logprobs(hidden: torch.Tensor, w_policy: torch.Tensor, w_ref: torch.Tensor, targets,
+                       temperature: float = 1.0, lengths=None, *, row_valid=None) -> DualLogprobs:
+    """Policy and reference log-probs of ``targets`` plus k3 KL and policy entropy, per token.
+
+    The two weight sets share ``hidden`` (in Tome the policy is the reference plus a merged
+    LoRA delta, mlx-impl/node.py:102-164).  k3 and entropy have no counterpart in the
+    reference node; they are defined by their closed forms.
+    """
+    lib = _lib.load_library()
+    dev, lead, h2, (wp, wr) = _check_fused_inputs(hidden, w_policy, w_ref)
+    if wp.stride(0) != wr.stride(0):
+        wr = wr.contiguous()
+        wp = wp.contiguous()
+    temperature = _check_temperature(temperature)
+    n, H = h2.shape
+    V = wp.shape[0]
+    tg = _as_i32(targets, n, dev, "targets")
+    rv = _row_valid(lead, n, lengths, row_valid, dev)
+    with torch.cuda.device(dev):
+        outs = [torch.empty(n, dtype=torch.float32, device=dev) for _ in range(4)]
+        ws_bytes = lib.tome_grpo_dual_workspace(n, H, V)
+        ws = _workspace(ws_bytes, dev)
+        _lib.check(lib.tome_grpo_dual(h2.data_ptr(), wp.data_ptr(), wr.data_ptr(), n, H, V,
+                                      h2.stride(0) if n > 1 else H, wp.stride(0), tg.data_ptr(), _ptr(rv),
+                                      temperature, outs[0].data_ptr(), outs[1].data_ptr(), outs[2].data_ptr(),
+                                      outs[3].data_ptr(), _ptr(ws), ws_bytes, _stream(dev)))
+    return DualLogprobs(*(o.reshape(lead) for o in outs))

@@ -1,0 +1,122 @@
+"""The reference-logprob entry of Tome's inference node, on the HIP kernels.
+
+Mirrors ``InferenceNodeServicer._process_ref_logprobs_batched``
+(mlx-impl/node.py:391-461): same name, arguments, in-place mutation of
+``results[p].completions[g].ref_log_probs`` and chunking by ``max_ref_batch_size``.
+The gRPC messages it walks (scheduler/proto/inference.proto:85-112) are mirrored
+as plain dataclasses; anything with the same attributes (``.tokens``,
+``.completions``, ``.ref_log_probs``) works, including the protobuf classes.
+"""
+from __future__ import annotations
+
+import logging
+import time
+from dataclasses import dataclass, field
+from typing import Any, Callable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from .logprob import fused_lmhead_logprobs, token_logprobs
+
+logger = logging.getLogger(__name__)
+
+
+@dataclass
+class Prompt:
+    """inference.proto:85-88"""
+    prompt_id: str = ""
+    tokens: List[int] = field(default_factory=list)
+
+
+@dataclass
+class Completion:
+    """inference.proto:108-112: one float per completion token in both lists."""
+    tokens: List[int] = field(default_factory=list)
+    log_probs: List[float] = field(default_factory=list)
+    ref_log_probs: List[float] = field(default_factory=list)
+
+
+@dataclass
+class PromptRollout:
+    """inference.proto:103-106"""
+    prompt_id: str = ""
+    completions: List[Completion] = field(default_factory=list)
+
+
+class RefLogprobServicer:
+    """The slice of InferenceNodeServicer (mlx-impl/node.py:49-100) that the ref-logprob path uses.
+
+    ``reference_model(full_ids, cache=None)`` follows Qwen3.__call__ (mlx-impl/model.py:522-540):
+    it takes int64 token ids [B, L] on ``device`` and returns ``(logits [B, L, V], cache)``.
+
+    If ``lm_head_weight`` ([V, H] bf16) is given, ``reference_model`` must instead return the
+    final, normalised hidden states ``(hidden [B, L, H] bf16, cache)``; only the completion rows
+    are then pushed through the fused lm_head + log-softmax kernel, so logits for prompt and
+    padding rows (which the reference computes at node.py:443 and discards at :449) are never
+    formed.
+    """
+
+    def __init__(self, reference_model: Callable[..., Any], device: torch.device | str = "cuda:0",
+                 max_ref_batch_size: int = 32, lm_head_weight: Optional[torch.Tensor] = None):
+        self.reference_model = reference_model
+        self.device = torch.device(device)
+        self.max_ref_batch_size = max_ref_batch_size     # node.py:58
+        self.lm_head_weight = lm_head_weight
+        self.last_ref_tokens = 0
+        self.last_ref_seconds = 0.0
+
+    async def _process_ref_logprobs_batched(self, prompts: Sequence, results: Sequence, G: int,
+                                            temperature: float = 1.0) -> None:
+        """Compute reference-model log-probs of every completion token, batched, without KV cache."""
+        self.process_ref_logprobs_batched(prompts, results, G, temperature)
+
+    def process_ref_logprobs_batched(self, prompts: Sequence, results: Sequence, G: int,
+                                     temperature: float = 1.0) -> None:
+        """Synchronous body of ``_process_ref_logprobs_batched`` (the reference's coroutine has no awaits)."""
+        t0 = time.perf_counter()
+        all_work = []                                                     # node.py:409-414
+        for p_idx, p in enumerate(prompts):
+            p_toks = list(p.tokens)
+            for g in range(G):
+                all_work.append((p_idx, g, p_toks, list(results[p_idx].completions[g].tokens)))
+
+        num_toks = 0
+        temp = temperature or 1.0                                         # node.py:451
+        for c0 in range(0, len(all_work), self.max_ref_batch_size):      # node.py:419-421
+            chunk = all_work[c0:c0 + self.max_ref_batch_size]
+            seqs = [p + c[:-1] if c else p for _, _, p, c in chunk]      # node.py:427-437
+            max_len = max(len(s) for s in seqs)
+            ids = np.zeros((len(chunk), max_len), dtype=np.int64)        # right-pad with id 0, node.py:440
+            targets = np.zeros((len(chunk), max_len), dtype=np.int32)
+            valid = np.zeros((len(chunk), max_len), dtype=np.int32)
+            spans = []
+            for i, (s, (_, _, p_toks, c_toks)) in enumerate(zip(seqs, chunk)):
+                ids[i, :len(s)] = s
+                if c_toks:                                               # rows p_len-1 .. p_len-2+len(c), node.py:449
+                    lo = len(p_toks) - 1
+                    if lo < 0:
+                        raise ValueError("a prompt needs at least one token to score its completion")
+                    targets[i, lo:lo + len(c_toks)] = c_toks
+                    valid[i, lo:lo + len(c_toks)] = 1
+                    spans.append((i, lo, len(c_toks)))
+            if not spans:
+                continue
+            full_ids = torch.from_numpy(ids).to(self.device)
+            out, _ = self.reference_model(full_ids, cache=None)           # node.py:443
+            tg = torch.from_numpy(targets).to(self.device)
+            rv = torch.from_numpy(valid).to(self.device)
+            if self.lm_head_weight is None:
+                lps = token_logprobs(out, tg, temp, row_valid=rv).lp
+            else:
+                lps = fused_lmhead_logprobs(out, self.lm_head_weight, tg, temp, row_valid=rv).lp
+            host = lps.cpu().numpy()                                      # one sync + one copy per chunk (node.py:456)
+            for i, lo, n in spans:
+                p_idx, g = chunk[i][0], chunk[i][1]
+                results[p_idx].completions[g].ref_log_probs.extend(host[i, lo:lo + n].tolist())  # node.py:458
+                num_toks += n
+
+        elapsed = time.perf_counter() - t0
+        self.last_ref_tokens, self.last_ref_seconds = num_toks, elapsed
+        logger.info("Ref log-probs non-KV batched completed: %d tokens in %.2fs (%.1f tok/s)",
+                    num_toks, elapsed, num_toks / elapsed if elapsed > 0 else 0.0)
