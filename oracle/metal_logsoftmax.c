@@ -126,8 +126,12 @@ int tome_oracle_local_compute_logprobs(const void* logits, int dtype, int64_t ro
         const char* in_row = (const char*)logits + row * V * (dtype == 0 ? 4 : 2);
         float m = -INFINITY;
         for (int64_t j = 0; j < V; ++j) m = fmaxf(m, load_elem(in_row, dtype, j) / temp);
-        float s = 0.0f;
-        for (int64_t j = 0; j < V; ++j) s += expf(load_elem(in_row, dtype, j) / temp - m);
+        /* fp32 sum over 16 interleaved partials, as a vectorised reduction would take it */
+        float part[16] = {0};
+        for (int64_t j = 0; j < V; ++j) part[j & 15] += expf(load_elem(in_row, dtype, j) / temp - m);
+        for (int w = 8; w > 0; w >>= 1)
+            for (int l = 0; l < w; ++l) part[l] += part[l + w];
+        const float s = part[0];
         out_lp[row] = load_elem(in_row, dtype, ids[row]) / temp - (m + logf(s));
     }
     return 0;

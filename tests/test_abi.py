@@ -1,0 +1,93 @@
+"""The C-ABI library loads, exports everything include/tome_logprob.h declares, and rejects bad
+arguments on the host before any GPU work (so these run without a GPU)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import tome_amd
+from tome_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tome_logprob.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tome_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    names = declared_functions()
+    assert "tome_row_logprob" in names and "tome_fused_lmhead_logprob" in names and "tome_grpo_dual" in names
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(tome_amd.lib_path())
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert tome_amd.load_library().tome_abi_version() == 1
+
+
+def test_header_cites_reference_for_each_entry_point():
+    text = open(HEADER).read()
+    for ref in ("mlx-impl/node.py:400-404", "mlx-impl/model.py:77-89", "mlx-impl/model.py:538"):
+        assert ref in text
+
+
+def test_strerror_and_codes():
+    lib = tome_amd.load_library()
+    assert lib.tome_strerror(0) == b"ok"
+    for code in range(-7, 0):
+        assert lib.tome_strerror(code) not in (b"ok", b"unknown error code")
+    assert lib.tome_strerror(-99) == b"unknown error code"
+
+
+def test_workspace_queries():
+    lib = tome_amd.load_library()
+    assert lib.tome_row_logprob_workspace(4096, 151936) == 0          # one workgroup per row
+    small = lib.tome_row_logprob_workspace(64, 151936)
+    assert small > 0 and small % 256 == 0
+    assert lib.tome_row_logprob_workspace(0, 151936) == 0
+    one = lib.tome_fused_lmhead_logprob_workspace(4096, 1024, 151936)
+    two = lib.tome_grpo_dual_workspace(4096, 1024, 151936)
+    assert 0 < one < two and one % 256 == 0
+
+
+def test_argument_checks_run_on_host():
+    """Every call below must return before touching the GPU (pointers are fake but non-NULL)."""
+    lib = tome_amd.load_library()
+    P = 0x1000  # 16-byte aligned dummy
+    row = lambda **k: lib.tome_row_logprob(k.get("logits", P), k.get("dtype", 1), k.get("rows", 4), k.get("V", 64),
+                                           k.get("stride", 64), k.get("targets", P), None, k.get("T", 1.0),
+                                           k.get("lp", P), None, None, None, None, 0, None)
+    assert row(dtype=7) == -2
+    assert row(V=0) == -3 and row(rows=-1) == -3 and row(stride=63) == -3
+    assert row(T=0.0) == -5 and row(T=-1.0) == -5 and row(T=float("nan")) == -5 and row(T=float("inf")) == -5
+    assert row(logits=None) == -1 and row(targets=None) == -1
+    assert row(lp=None) == -1                      # no output requested at all
+    assert row(rows=0) == 0                        # empty batch is a no-op
+    assert row(rows=64, V=151936, stride=151936) == -4   # split rows need a workspace
+    assert row(logits=P + 1) == -6
+    fused = lambda **k: lib.tome_fused_lmhead_logprob(k.get("h", P), k.get("w", P), k.get("n", 8), k.get("H", 64),
+                                                      k.get("V", 100), k.get("hs", 64), k.get("ws", 64), P, None,
+                                                      k.get("T", 1.0), k.get("lp", P), None, None, None, None, 0, None)
+    assert fused(H=0) == -3 and fused(hs=32) == -3 and fused(T=0.0) == -5
+    assert fused(H=60, hs=60, ws=60) == -6 and fused(h=P + 2) == -6
+    assert fused(h=None) == -1 and fused(n=0) == 0
+    assert fused(n=1 << 20, H=4096, hs=4096, ws=4096) == -3          # > 4 GiB of hidden
+    assert fused() == -4                                             # workspace missing
+    dual = lib.tome_grpo_dual(P, P, None, 8, 64, 100, 64, 64, P, None, 1.0, P, P, P, P, None, 0, None)
+    assert dual == -1
+
+
+def test_check_maps_codes_to_exceptions():
+    with pytest.raises(ValueError):
+        _lib.check(-3)
+    with pytest.raises(tome_amd.TomeError) as e:
+        _lib.check(-4)
+    assert e.value.code == -4
+    _lib.check(0)

@@ -1,0 +1,212 @@
+"""Pins the CPU oracle: golden vectors, closed forms, brute force, independent library routines.
+
+Each check is chosen so that a plausible slip (dropped max shift, wrong sign, temperature applied
+to one term only, transposed weight, off-by-one gather) fails it.
+"""
+import math
+
+import numpy as np
+import pytest
+import scipy.special
+import scipy.stats
+
+import oracle
+from oracle import cport
+from oracle.logprob_oracle import _brute_logprob
+from golden_util import V_QWEN3, load, seeded_case
+
+G = load()
+
+
+# ---- golden vectors ---------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["s0", "s1", "s2"])
+def test_golden_small_bruteforce(name):
+    x, t, T = G[f"{name}_x"], G[f"{name}_t"], float(G[f"{name}_T"])
+    np.testing.assert_allclose(oracle.logprob_rows(x, t, T), G[f"{name}_lp"], atol=1e-12)
+    np.testing.assert_allclose(oracle.lse_rows(x, T), G[f"{name}_lse"], atol=1e-12)
+    np.testing.assert_allclose(oracle.entropy_rows(x, T), G[f"{name}_ent"], atol=1e-12)
+
+
+def test_golden_bf16_spike_rows():
+    b, t = G["b0_bits"], G["b0_t"]
+    np.testing.assert_allclose(oracle.logprob_rows(b, t, 1.0), G["b0_lp"], atol=1e-12)
+    np.testing.assert_allclose(oracle.entropy_rows(b, 1.0), G["b0_ent"], atol=1e-11)
+    np.testing.assert_array_equal(oracle.argmax_rows(b), G["b0_argmax"])
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c2t"])
+def test_golden_full_vocab(name):
+    x, t, T, exp = seeded_case(G, name)
+    np.testing.assert_allclose(oracle.logprob_rows(x, t, T), exp["lp"], atol=1e-11)
+    np.testing.assert_allclose(oracle.lse_rows(x, T), exp["lse"], atol=1e-11)
+    np.testing.assert_allclose(oracle.entropy_rows(x, T), exp["ent"], atol=1e-10)
+    np.testing.assert_array_equal(oracle.argmax_rows(x), exp["argmax"])
+    # fp32 restatement of node.py:400-404 agrees with the closed form far inside the parity tolerance
+    np.testing.assert_allclose(oracle.local_compute_logprobs_f32(x, t, T), exp["lp"], atol=2e-5)
+    np.testing.assert_allclose(cport.local_compute_logprobs_c(x, t, T), exp["lp"], atol=5e-5)
+
+
+def test_golden_lmhead():
+    h, w, t, T = G["f0_h"], G["f0_w"], G["f0_t"], float(G["f0_T"])
+    st = oracle.lmhead_stats(h, w, t, T, row_chunk=7)
+    np.testing.assert_allclose(st["lp"], G["f0_lp"], atol=1e-12)
+    np.testing.assert_allclose(st["lse"], G["f0_lse"], atol=1e-12)
+    np.testing.assert_allclose(st["entropy"], G["f0_ent"], atol=1e-12)
+    np.testing.assert_array_equal(st["argmax"], G["f0_argmax"])
+    assert (st["top1"] >= st["top2"]).all()
+
+
+# ---- closed forms -----------------------------------------------------------------------------
+def test_all_equal_row_is_minus_log_v():
+    x = np.full((2, V_QWEN3), -7.5, dtype=np.float32)
+    np.testing.assert_allclose(oracle.logprob_rows(x, [0, V_QWEN3 - 1], 0.6), -math.log(V_QWEN3), atol=1e-12)
+    assert abs(-math.log(V_QWEN3) - (-11.9312147)) < 1e-6      # ln 128 + ln 1187
+    np.testing.assert_allclose(oracle.entropy_rows(x, 0.6), math.log(V_QWEN3), atol=1e-10)
+
+
+@pytest.mark.parametrize("c,T", [(15.0, 1.0), (15.0, 0.7), (3.0, 2.0)])
+def test_single_spike_closed_form(c, T):
+    V = V_QWEN3
+    x = np.zeros((1, V), dtype=np.float32)
+    x[0, 4242] = c
+    want_spike = -math.log1p((V - 1) * math.exp(-c / T))
+    np.testing.assert_allclose(oracle.logprob_rows(x, [4242], T), want_spike, atol=1e-12)
+    np.testing.assert_allclose(oracle.logprob_rows(x, [0], T), want_spike - c / T, atol=1e-12)
+
+
+def test_shift_invariance_and_temperature_identity():
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((5, 1000)) * 4
+    t = rng.integers(0, 1000, size=5)
+    base = oracle.logprob_rows(x, t, 0.7)
+    np.testing.assert_allclose(oracle.logprob_rows(x + 123.0, t, 0.7), base, atol=1e-10)
+    np.testing.assert_allclose(oracle.logprob_rows(x / 0.7, t, 1.0), base, atol=1e-10)
+    # a large offset must not overflow (the max shift is there)
+    assert np.isfinite(oracle.lse_rows(x + 5000.0)).all()
+
+
+def test_bruteforce_tiny_rows():
+    rng = np.random.default_rng(1)
+    for V in (1, 2, 3, 16):
+        x = rng.standard_normal((4, V)) * 3
+        for r in range(4):
+            for t in range(V):
+                for T in (1.0, 0.5):
+                    assert abs(oracle.logprob_rows(x[r:r + 1], [t], T)[0] - _brute_logprob(x[r], t, T)) < 1e-12
+    # probabilities of a row sum to one
+    lp_all = oracle.full_log_softmax64(x, 0.8)
+    np.testing.assert_allclose(np.exp(lp_all).sum(-1), 1.0, atol=1e-12)
+
+
+def test_against_scipy_and_torch_routines():
+    import torch
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal((6, 5000)) * 3).astype(np.float32)
+    t = rng.integers(0, 5000, size=6)
+    T = 1.7
+    z = x.astype(np.float64) / T
+    np.testing.assert_allclose(oracle.lse_rows(x, T), scipy.special.logsumexp(z, axis=-1), atol=1e-12)
+    ls = scipy.special.log_softmax(z, axis=-1)
+    np.testing.assert_allclose(oracle.full_log_softmax64(x, T), ls, atol=1e-12)
+    np.testing.assert_allclose(oracle.logprob_rows(x, t, T), ls[np.arange(6), t], atol=1e-12)
+    np.testing.assert_allclose(oracle.entropy_rows(x, T), scipy.stats.entropy(np.exp(ls), axis=-1), atol=1e-10)
+    tl = torch.log_softmax(torch.from_numpy(z), -1).numpy()
+    np.testing.assert_allclose(oracle.full_log_softmax64(x, T), tl, atol=1e-12)
+
+
+def test_entropy_bounds_and_limits():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((8, 777)) * 5
+    h = oracle.entropy_rows(x, 1.0)
+    assert (h >= 0).all() and (h <= math.log(777) + 1e-12).all()
+    onehot = np.zeros((1, 50)); onehot[0, 7] = 80.0
+    assert oracle.entropy_rows(onehot)[0] < 1e-20 + 1e-9
+    # higher temperature flattens the distribution
+    assert (oracle.entropy_rows(x, 2.0) > h).all()
+
+
+def test_k3_properties():
+    rng = np.random.default_rng(4)
+    lp = -rng.random(100) * 5
+    ref = lp + rng.standard_normal(100) * 0.3
+    k = oracle.k3(lp, ref)
+    assert (k >= 0).all()
+    assert (oracle.k3(lp, lp) == 0).all()
+    d = 1e-3
+    assert abs(oracle.k3(np.array([-1.0]), np.array([-1.0 + d]))[0] - (d * d / 2 + d ** 3 / 6)) < 1e-12
+    np.testing.assert_allclose(k, np.exp(ref - lp) - (ref - lp) - 1, atol=1e-12)
+    # sign convention: d = ref_lp - lp (k3 estimates KL(pi || pi_ref) at a sample from pi)
+    assert abs(oracle.k3(np.array([0.0]), np.array([-1.0]))[0] - (math.exp(-1) + 1 - 1)) < 1e-12
+
+
+def test_argmax_first_max_wins():
+    x = np.zeros((3, 100), dtype=np.float32)
+    x[0, [5, 50]] = 2.0
+    x[1, [99, 0]] = 1.0
+    x[2, 60] = 3.0
+    assert oracle.argmax_rows(x).tolist() == [5, 0, 60]
+    assert oracle.argmax_rows(oracle.bf16_round(x)).tolist() == [5, 0, 60]
+
+
+def test_bf16_conversions():
+    import torch
+    rng = np.random.default_rng(5)
+    x = np.concatenate([rng.standard_normal(10000).astype(np.float32) * 100,
+                        np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.4e38, 1e-40], dtype=np.float32)])
+    bits = oracle.bf16_round(x)
+    want = torch.from_numpy(x).to(torch.bfloat16)
+    np.testing.assert_array_equal(bits, want.view(torch.int16).numpy().view(np.uint16))   # round-to-nearest-even
+    np.testing.assert_array_equal(oracle.bf16_to_f32(bits), want.float().numpy())
+
+
+def test_lmhead_orientation_and_bruteforce():
+    """logits = hidden @ W.T with W [V, H] (model.py:538); a transposed operand fails this."""
+    rng = np.random.default_rng(6)
+    n, H, V = 3, 5, 7
+    h = oracle.bf16_round(rng.standard_normal((n, H)).astype(np.float32))
+    w = oracle.bf16_round(rng.standard_normal((V, H)).astype(np.float32))
+    hf, wf = oracle.bf16_to_f32(h).astype(np.float64), oracle.bf16_to_f32(w).astype(np.float64)
+    logits = oracle.lmhead_logits64(h, w)
+    assert logits.shape == (n, V)
+    for r in range(n):
+        for v in range(V):
+            assert abs(logits[r, v] - math.fsum(hf[r, k] * wf[v, k] for k in range(H))) < 1e-12
+    t = np.array([0, 6, 3])
+    st = oracle.lmhead_stats(h, w, t, 0.5, row_chunk=2)
+    np.testing.assert_allclose(st["lp"], oracle.logprob_rows(logits, t, 0.5), atol=1e-12)
+    np.testing.assert_array_equal(st["argmax"], oracle.argmax_rows(logits))
+
+
+# ---- restatements of the reference's own arithmetic ------------------------------------------------
+def test_reference_kernel_check_restated():
+    """tests/test_logprob_comparison.py:84-102: bf16 [1, 151936] ~ N(0, 1), T = 1, kernel vs
+    `logits - logsumexp(logits)` in bf16, max abs diff < 5e-3."""
+    rng = np.random.default_rng(7)
+    bits = oracle.bf16_round(rng.standard_normal((1, V_QWEN3)).astype(np.float32))
+    lse_b = oracle.bf16_to_f32(oracle.bf16_round(oracle.lse_rows(bits).astype(np.float32)))
+    expected = oracle.bf16_to_f32(oracle.bf16_round(oracle.bf16_to_f32(bits) - lse_b[:, None]))
+    for impl in (oracle.fused_log_softmax_f32, cport.metal_log_softmax):
+        actual = oracle.bf16_to_f32(impl(bits, 1.0))
+        assert np.abs(actual - expected).max() < 5e-3
+
+
+@pytest.mark.parametrize("V", [4096, 4097, 8192 + 384, V_QWEN3, 166144, 5])
+def test_metal_restatement_tails(V):
+    """Tail handling of model.py:17-20,34-36: V % 4096 in {0, 1, 384}, V < one block."""
+    rng = np.random.default_rng(V)
+    x = (rng.standard_normal((2, V)) * 2).astype(np.float32)
+    for T in (1.0, 0.7):
+        want = oracle.full_log_softmax64(x, T)
+        np.testing.assert_allclose(cport.metal_log_softmax(x, T), want, atol=2e-5)
+        np.testing.assert_allclose(oracle.fused_log_softmax_f32(x, T), want, atol=2e-5)
+
+
+def test_local_compute_logprobs_restatement_divides_by_temp():
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((4, 3000)) * 3).astype(np.float32)
+    t = rng.integers(0, 3000, size=4)
+    for T in (1.0, 0.7, 1.9):
+        np.testing.assert_allclose(oracle.local_compute_logprobs_f32(x, t, T), oracle.logprob_rows(x, t, T), atol=1e-5)
+    # bf16 input is upcast exactly first (node.py:401)
+    b = oracle.bf16_round(x)
+    np.testing.assert_allclose(oracle.local_compute_logprobs_f32(b, t, 0.7), oracle.logprob_rows(b, t, 0.7), atol=1e-5)
