@@ -74,6 +74,100 @@ __device__ __forceinline__ u32x4 ld16(__amdgpu_buffer_rsrc_t r, uint32_t lane_of
   return __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, uniform_off, 0);
 }
 
+
+// Fold one wave tile of logits (kNBV x kNBT blocks of 32x32 accumulators) into the per-token
+// running states.  Accumulator element e of block i holds vocab row
+//   vw0 + i*32 + 8*(e/4) + 4*lh + e%4        (vw0 = first vocab row of this wave's tile)
+// for the token this lane owns in block column j.
+template <bool ENT>
+__device__ __forceinline__ void fold_tile(f32x16 (&acc)[kNBV][kNBT], RowStat (&st)[kNBT], float (&tx)[kNBT],
+                                          const int (&tgt)[kNBT], int vw0, int lh, bool partial_tile, int V,
+                                          float scale) {
+  if (partial_tile) {  // last vocab tile: rows past V do not exist
+#pragma unroll
+    for (int i = 0; i < kNBV; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const bool dead = vw0 + 4 * lh + i * 32 + 8 * (e / 4) + (e % 4) >= V;
+#pragma unroll
+        for (int j = 0; j < kNBT; ++j) acc[i][j][e] = dead ? -INFINITY : acc[i][j][e];
+      }
+  }
+#pragma unroll
+  for (int j = 0; j < kNBT; ++j) {
+    // Target capture: rare (one tile in V/256 per token), so behind a wave-uniform test.
+    const int rel = tgt[j] - vw0;
+    const bool mine = tgt[j] >= 0 && rel >= 0 && rel < kWaveV && ((rel >> 2) & 1) == lh;
+    if (__any(mine)) {
+      const int want = mine ? ((rel >> 5) * 16 + ((rel & 31) >> 3) * 4 + (rel & 3)) : -1;
+#pragma unroll
+      for (int i = 0; i < kNBV; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) tx[j] = (want == i * 16 + e) ? acc[i][j][e] : tx[j];
+    }
+    float bm[kNBV];  // per 32-row block maximum
+#pragma unroll
+    for (int i = 0; i < kNBV; ++i) {
+      float m = acc[i][j][0];
+#pragma unroll
+      for (int e = 1; e < 16; e += 2) m = fmaxf(m, fmaxf(acc[i][j][e], e + 1 < 16 ? acc[i][j][e + 1] : acc[i][j][e]));
+      bm[i] = m;
+    }
+    float cm = st[j].mx;
+    int bi = st[j].bi;
+#pragma unroll
+    for (int i = 0; i < kNBV; ++i) {
+      const bool up = bm[i] > cm;
+      bi = up ? (vw0 + i * 32) : bi;  // first row of the 32-row block
+      cm = fmaxf(cm, bm[i]);
+    }
+    const float resc = fast_exp2((st[j].mx - cm) * scale);
+    const float m = cm * scale;
+    float s0 = st[j].s * resc, s1 = 0.f, w0 = ENT ? st[j].w * resc : 0.f, w1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < kNBV; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; e += 2) {
+        const float x0 = acc[i][j][e], x1 = acc[i][j][e + 1];
+        const float e0 = fast_exp2(fmaf(x0, scale, -m));
+        const float e1 = fast_exp2(fmaf(x1, scale, -m));
+        s0 += e0;
+        s1 += e1;
+        if constexpr (ENT) {
+          w0 = fmaf(fmaxf(x0, kMaxFloor) * scale, e0, w0);
+          w1 = fmaf(fmaxf(x1, kMaxFloor) * scale, e1, w1);
+        }
+      }
+    st[j].mx = cm;
+    st[j].bi = bi;
+    st[j].s = s0 + s1;
+    if constexpr (ENT) st[j].w = w0 + w1;
+  }
+}
+
+// Merge the two lane halves that share a token and write one partial per (token, part).
+__device__ __forceinline__ void write_partials(RowStat (&st)[kNBT], float (&tx)[kNBT], FusedPartial* partials,
+                                               int p0, int n_valid, int part, int n_parts, int l32, int lh,
+                                               float scale) {
+#pragma unroll
+  for (int j = 0; j < kNBT; ++j) {
+    stat_wave_step<5>(st[j], scale);
+    const float txo = wave_exchange<5>(tx[j]);
+    tx[j] = fmaxf(tx[j], txo);
+    const int p = p0 + j * 32 + l32;
+    if (lh == 0 && p < n_valid) {
+      FusedPartial out;
+      out.mx = st[j].mx;
+      out.s = st[j].s;
+      out.w = st[j].w;
+      out.tx = tx[j];
+      out.bi = st[j].bi;
+      out.pad[0] = out.pad[1] = out.pad[2] = 0;
+      partials[(int64_t)p * n_parts + part] = out;
+    }
+  }
+}
+
 template <bool ENT>
 __global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) {
   __shared__ __attribute__((aligned(16))) char lds[(kBV + kBT) * kPitch];
@@ -186,90 +280,207 @@ __global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) 
       }
     }
 
-    // ---- epilogue: fold this tile's logits into the per-token states ----------------------
-    // Accumulator element e of block i holds vocab row  v0 + wave_v*128 + i*32 + 8*(e/4) + 4*lh + e%4.
-    const int vbase = v0 + wave_v * kWaveV + 4 * lh;
-    if (v0 + kBV > a.V) {  // last, partial vocab tile: rows past V do not exist
+    fold_tile<ENT>(acc, st, tx, tgt, v0 + wave_v * kWaveV, lh, v0 + kBV > a.V, a.V, a.scale);
+  }
+
+  write_partials(st, tx, a.partials, t0 + wave_t * kWaveT, n_valid, split * kPartsPerSplit + wave_v,
+                 a.n_splits * kPartsPerSplit, l32, lh, a.scale);
+}
+
+
+// ===============================================================================================
+// Fast path (H % 64 == 0): 512 lanes, 256 x 256 tile, K slabs DMA'd straight into LDS.
+//
+//   * 8 waves as 2 (vocab) x 4 (token); the per-wave tile is still 128 vocab x 64 tokens, so
+//     fold_tile / write_partials and the partial layout are shared with the generic kernel.
+//   * global_load_lds_dwordx4: every lane fetches 16 bytes and the wave's 1 KB lands contiguously
+//     in LDS, bypassing registers.  No staging registers are needed, which leaves room to
+//     double-buffer the MFMA fragments (LDS reads of sub-step k+1 fly during the MFMAs of k).
+//   * LDS holds two 64 KB slabs (W 256 rows + hidden 256 rows, 128 bytes per row, no padding).
+//     The slab for step s+1 is requested at the start of step s and waited for at its end: one
+//     barrier per slab, latency hidden behind 32 MFMAs per wave.  Steps run across vocab-tile
+//     boundaries, so the first slab of the next tile streams in during the epilogue.
+//   * Bank conflicts are avoided by an XOR swizzle instead of padding (DMA writes are dense).
+//     The LDS has 64 four-byte banks, so a 16-lane phase of a 128-bit read is conflict-free when
+//     its 16 rows hit 16 different 16-byte bank groups.  Row r covers groups 8*(r&1) .. +7, so
+//     chunk c of row r is stored at chunk position c ^ ((r >> 1) & 7); the lane that DMA-writes
+//     position p of row r fetches global chunk p ^ ((r >> 1) & 7).
+// ===============================================================================================
+constexpr int k2BV = 256, k2BT = 256, k2WG = 512;
+constexpr int k2RowBytes = kBK * 2;                    // 128
+constexpr int k2SlabBytes = (k2BV + k2BT) * k2RowBytes;  // 65536
+constexpr int k2LdsBytes = 2 * k2SlabBytes;
+constexpr int k2LdsTotal = k2LdsBytes;
+constexpr int k2Loads = k2BV * 8 / k2WG;               // DMA instructions per lane per operand per slab (4)
+
+__device__ __forceinline__ void dma16(const char* gptr, char* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(gptr),
+                                   reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(
+                                       reinterpret_cast<__attribute__((address_space(3))) char*>(
+                                           (__attribute__((address_space(3))) char*)lds_wave_base)),
+                                   16, 0, 0);
+}
+
+template <bool ENT>
+__global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  int bid = blockIdx.x;
+  const int nwg = gridDim.x;
+  if ((nwg & 7) == 0) bid = (bid & 7) * (nwg >> 3) + (bid >> 3);  // contiguous logical ids per XCD
+  const int ttile = bid / a.n_splits;
+  const int split = bid % a.n_splits;
+  const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
+  const int t0 = ttile * k2BT;
+  if (t0 >= n_valid) return;
+  const int vt0 = (int)((int64_t)split * a.n_vtiles / a.n_splits);
+  const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / a.n_splits);
+  if (vt0 >= vt1) return;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wave_v = wave & 1, wave_t = wave >> 1;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  // ---- DMA assignment: instruction j of wave w fills LDS rows (j*8 + w)*8 .. +7 of an operand ----
+  // All address arithmetic is incremental: per-lane pointers advance by one slab (128 bytes) per
+  // step and are rebased at vocab-tile changes, so a step carries no multiplies or divides.
+  const int dr = lane >> 3;                                   // row inside the 8-row group
+  const int dc = (lane & 7) ^ (((wave & 1) << 2) | (dr >> 1));  // global chunk: position ^ ((row >> 1) & 7)
+  const char* pa[k2Loads];  // next W slab to request, per DMA instruction
+  const char* pb[k2Loads];  // next hidden slab
+  auto point_a = [&](int vt) {  // rows past V (last tile only) read the last row; masked in the epilogue
+#pragma unroll
+    for (int j = 0; j < k2Loads; ++j) {
+      int64_t v = (int64_t)vt * k2BV + (j * 8 + wave) * 8 + dr;
+      v = v < a.V ? v : a.V - 1;
+      pa[j] = a.weight + v * a.weight_stride_b + dc * 16;
+    }
+  };
+  point_a(vt0);
+#pragma unroll
+  for (int j = 0; j < k2Loads; ++j) {
+    int p = t0 + (j * 8 + wave) * 8 + dr;
+    p = p < n_valid ? p : n_valid - 1;
+    const int tok = a.row_index ? a.row_index[p] : p;
+    pb[j] = a.hidden + (int64_t)tok * a.hidden_stride_b + dc * 16;
+  }
+
+  RowStat st[kNBT];
+  float tx[kNBT];
+  int tgt[kNBT];
+#pragma unroll
+  for (int bt = 0; bt < kNBT; ++bt) {
+    st[bt] = stat_identity();
+    tx[bt] = -INFINITY;
+    const int p = t0 + wave_t * kWaveT + bt * 32 + l32;
+    int t = -1;
+    if (p < n_valid) t = a.targets[a.row_index ? a.row_index[p] : p];
+    tgt[bt] = (t >= 0 && t < a.V) ? t : -1;
+  }
+
+  // ---- fragment read offsets inside a slab (swizzled) --------------------------------------------
+  const int x7 = (l32 >> 1) & 7;
+  int swz[kBK / 16];
+#pragma unroll
+  for (int ks = 0; ks < kBK / 16; ++ks) swz[ks] = ((ks * 2 + lh) ^ x7) * 16;
+  const int rdA = (wave_v * kWaveV + l32) * k2RowBytes;
+  const int rdB = k2BV * k2RowBytes + (wave_t * kWaveT + l32) * k2RowBytes;
+
+  const int nk = a.H / kBK;
+  const int64_t slab_rewind = (int64_t)nk * k2RowBytes;
+  int i_kt = 0, i_vt = vt0;  // slab the next `issue` will request
+  int buf = 0;               // LDS slab that request lands in
+
+  auto issue = [&]() {
+    char* dst = smem + buf * k2SlabBytes + wave * 1024;
+#pragma unroll
+    for (int j = 0; j < k2Loads; ++j) dma16(pa[j], dst + j * 8192);
+#pragma unroll
+    for (int j = 0; j < k2Loads; ++j) dma16(pb[j], dst + k2BV * k2RowBytes + j * 8192);
+    buf ^= 1;
+    if (++i_kt < nk) {
+#pragma unroll
+      for (int j = 0; j < k2Loads; ++j) {
+        pa[j] += k2RowBytes;
+        pb[j] += k2RowBytes;
+      }
+    } else {
+      i_kt = 0;
+      ++i_vt;
+#pragma unroll
+      for (int j = 0; j < k2Loads; ++j) pb[j] -= slab_rewind - k2RowBytes;
+      if (i_vt < vt1) point_a(i_vt);
+    }
+  };
+
+  issue();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  int cur = 0;
+  for (int vt = vt0; vt < vt1; ++vt) {
+    f32x16 acc[kNBV][kNBT];
+#pragma unroll
+    for (int i = 0; i < kNBV; ++i)
+#pragma unroll
+      for (int j = 0; j < kNBT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    for (int kt = 0; kt < nk; ++kt) {
+      // Request the next slab (possibly the first slab of the next vocab tile, which then
+      // streams in during the epilogue) before touching the current one.
+      if (i_vt < vt1) issue();
+
+      const char* slab = smem + cur * k2SlabBytes;
+      bf16x8 fa[2][kNBV], fb[2][kNBT];
 #pragma unroll
       for (int i = 0; i < kNBV; ++i)
+        fa[0][i] = *reinterpret_cast<const bf16x8*>(slab + rdA + i * 32 * k2RowBytes + swz[0]);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const bool dead = vbase + i * 32 + 8 * (e / 4) + (e % 4) >= a.V;
+      for (int j = 0; j < kNBT; ++j)
+        fb[0][j] = *reinterpret_cast<const bf16x8*>(slab + rdB + j * 32 * k2RowBytes + swz[0]);
 #pragma unroll
-          for (int j = 0; j < kNBT; ++j) acc[i][j][e] = dead ? -INFINITY : acc[i][j][e];
+      for (int ks = 0; ks < kBK / 16; ++ks) {
+        const int c = ks & 1, n = c ^ 1;
+        // Scheduling fences pin the software pipeline: the LDS reads of sub-step ks+1 are issued
+        // before the MFMAs of sub-step ks, which then cover their latency.  Left alone, the
+        // scheduler sinks every read next to its use and reuses one fragment register set.
+        __builtin_amdgcn_sched_barrier(0);
+        if (ks + 1 < kBK / 16) {
+#pragma unroll
+          for (int i = 0; i < kNBV; ++i)
+            fa[n][i] = *reinterpret_cast<const bf16x8*>(slab + rdA + i * 32 * k2RowBytes + swz[ks + 1]);
+#pragma unroll
+          for (int j = 0; j < kNBT; ++j)
+            fb[n][j] = *reinterpret_cast<const bf16x8*>(slab + rdB + j * 32 * k2RowBytes + swz[ks + 1]);
         }
-    }
-#pragma unroll
-    for (int j = 0; j < kNBT; ++j) {
-      // Target capture: rare (one tile in V/256 per token), so behind a wave-uniform test.
-      const int rel = tgt[j] - (v0 + wave_v * kWaveV);
-      const bool mine = tgt[j] >= 0 && rel >= 0 && rel < kWaveV && ((rel >> 2) & 1) == lh;
-      if (__any(mine)) {
-        const int want = mine ? ((rel >> 5) * 16 + ((rel & 31) >> 3) * 4 + (rel & 3)) : -1;
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < kNBV; ++i)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) tx[j] = (want == i * 16 + e) ? acc[i][j][e] : tx[j];
+          for (int j = 0; j < kNBT; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[c][i], fb[c][j], acc[i][j], 0, 0, 0);
       }
-      float bm[kNBV];  // per 32-row block maximum
-#pragma unroll
-      for (int i = 0; i < kNBV; ++i) {
-        float m = acc[i][j][0];
-#pragma unroll
-        for (int e = 1; e < 16; e += 2) m = fmaxf(m, fmaxf(acc[i][j][e], e + 1 < 16 ? acc[i][j][e + 1] : acc[i][j][e]));
-        bm[i] = m;
+
+      if (kt == nk - 1) {
+        const int v0 = vt * k2BV;
+#ifndef TOME_EXP_NOFOLD
+        fold_tile<ENT>(acc, st, tx, tgt, v0 + wave_v * kWaveV, lh, v0 + k2BV > a.V, a.V, a.scale);
+#else
+        for (int i = 0; i < kNBV; ++i) for (int j = 0; j < kNBT; ++j) st[j].s += acc[i][j][0] + v0;
+#endif
       }
-      float cm = st[j].mx;
-      int bi = st[j].bi;
-#pragma unroll
-      for (int i = 0; i < kNBV; ++i) {
-        const bool up = bm[i] > cm;
-        bi = up ? (v0 + wave_v * kWaveV + i * 32) : bi;  // first row of the 32-row block
-        cm = fmaxf(cm, bm[i]);
-      }
-      const float resc = fast_exp2((st[j].mx - cm) * a.scale);
-      const float m = cm * a.scale;
-      float s0 = st[j].s * resc, s1 = 0.f, w0 = ENT ? st[j].w * resc : 0.f, w1 = 0.f;
-#pragma unroll
-      for (int i = 0; i < kNBV; ++i)
-#pragma unroll
-        for (int e = 0; e < 16; e += 2) {
-          const float x0 = acc[i][j][e], x1 = acc[i][j][e + 1];
-          const float e0 = fast_exp2(fmaf(x0, a.scale, -m));
-          const float e1 = fast_exp2(fmaf(x1, a.scale, -m));
-          s0 += e0;
-          s1 += e1;
-          if constexpr (ENT) {
-            w0 = fmaf(fmaxf(x0, kMaxFloor) * a.scale, e0, w0);
-            w1 = fmaf(fmaxf(x1, kMaxFloor) * a.scale, e1, w1);
-          }
-        }
-      st[j].mx = cm;
-      st[j].bi = bi;
-      st[j].s = s0 + s1;
-      if constexpr (ENT) st[j].w = w0 + w1;
+      cur ^= 1;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next slab has landed
+      // Bare barrier (no fence): LDS reads of the current slab were consumed by the MFMAs above and
+      // the DMA writes are covered by the explicit wait, so nothing else needs draining.
+      __builtin_amdgcn_s_barrier();
     }
   }
 
-  // ---- merge the two lane halves that share a token, write one partial per token ----------
-#pragma unroll
-  for (int j = 0; j < kNBT; ++j) {
-    stat_wave_step<5>(st[j], a.scale);
-    const float txo = wave_exchange<5>(tx[j]);
-    tx[j] = fmaxf(tx[j], txo);
-    const int p = t0 + wave_t * kWaveT + j * 32 + l32;
-    if (lh == 0 && p < n_valid) {
-      const int part = split * kPartsPerSplit + wave_v;
-      FusedPartial out;
-      out.mx = st[j].mx;
-      out.s = st[j].s;
-      out.w = st[j].w;
-      out.tx = tx[j];
-      out.bi = st[j].bi;
-      out.pad[0] = out.pad[1] = out.pad[2] = 0;
-      a.partials[(int64_t)p * (a.n_splits * kPartsPerSplit) + part] = out;
-    }
-  }
+  write_partials(st, tx, a.partials, t0 + wave_t * kWaveT, n_valid, split * kPartsPerSplit + wave_v,
+                 a.n_splits * kPartsPerSplit, l32, lh, a.scale);
 }
 
 // ---- compaction of valid rows ----------------------------------------------------------------
@@ -383,10 +594,17 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
 }
 
 // ---- host side -----------------------------------------------------------------------------------
-static int fused_splits(int64_t n_tokens, int64_t V) {
-  const int64_t n_ttiles = (n_tokens + kBT - 1) / kBT;
-  const int64_t n_vtiles = (V + kBV - 1) / kBV;
-  int64_t s = (512 + n_ttiles - 1) / n_ttiles;  // ~2 resident workgroups on each of 256 CUs
+// The DMA kernel needs whole 64-wide K slabs and pays for 256-token tiles; short batches and
+// ragged H go to the generic kernel.
+static bool use_dma_kernel(int64_t n_tokens, int64_t H) { return H % kBK == 0 && n_tokens > kBT; }
+
+static int fused_splits(int64_t n_tokens, int64_t H, int64_t V) {
+  const bool dma = use_dma_kernel(n_tokens, H);
+  const int64_t bt = dma ? k2BT : kBT, bv = dma ? k2BV : kBV;
+  const int64_t slots = dma ? 256 : 512;  // resident workgroups on 256 CUs: 1 per CU (128 KB LDS) or 2
+  const int64_t n_ttiles = (n_tokens + bt - 1) / bt;
+  const int64_t n_vtiles = (V + bv - 1) / bv;
+  int64_t s = (slots + n_ttiles - 1) / n_ttiles;
   if (s > n_vtiles) s = n_vtiles;
   if (s < 1) s = 1;
   return (int)s;
@@ -395,13 +613,29 @@ static int fused_splits(int64_t n_tokens, int64_t V) {
 // Layout: [n_valid: 256 B][row_index: n_tokens int32, 256-aligned][partials per weight set].
 static size_t off_index() { return 256; }
 static size_t off_partials(int64_t n_tokens) { return 256 + (((size_t)n_tokens * 4 + 255) & ~(size_t)255); }
-static size_t partial_bytes(int64_t n_tokens, int64_t V) {
-  return (size_t)n_tokens * (size_t)fused_splits(n_tokens, V) * kPartsPerSplit * sizeof(FusedPartial);
+static size_t partial_bytes(int64_t n_tokens, int64_t H, int64_t V) {
+  return (size_t)n_tokens * (size_t)fused_splits(n_tokens, H, V) * kPartsPerSplit * sizeof(FusedPartial);
 }
 
 size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights) {
-  (void)H;
-  return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, V);
+  return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, H, V);
+}
+
+template <bool ENT>
+static void launch_main(const FusedArgs& a, bool dma, hipStream_t stream) {
+  if (dma) {
+    static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
+    if (!attr_set) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_lmhead_dma_kernel<ENT>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, k2LdsTotal);
+      attr_set = true;
+    }
+    hipLaunchKernelGGL(fused_lmhead_dma_kernel<ENT>, dim3((unsigned)(a.n_ttiles * a.n_splits)), dim3(k2WG),
+                       k2LdsTotal, stream, a);
+  } else {
+    hipLaunchKernelGGL(fused_lmhead_kernel<ENT>, dim3((unsigned)(a.n_ttiles * a.n_splits)), dim3(kFusedWG), 0,
+                       stream, a);
+  }
 }
 
 hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w1, int64_t n_tokens, int64_t H,
@@ -435,22 +669,23 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w
   a.n_tokens = (int)n_tokens;
   a.H = (int)H;
   a.V = (int)V;
-  a.n_vtiles = (int)((V + kBV - 1) / kBV);
-  a.n_splits = fused_splits(n_tokens, V);
-  a.n_ttiles = (int)((n_tokens + kBT - 1) / kBT);
+  const bool dma = use_dma_kernel(n_tokens, H);
+  const int64_t bt = dma ? k2BT : kBT, bv = dma ? k2BV : kBV;
+  a.n_vtiles = (int)((V + bv - 1) / bv);
+  a.n_splits = fused_splits(n_tokens, H, V);
+  a.n_ttiles = (int)((n_tokens + bt - 1) / bt);
   a.scale = kLog2e / temperature;
-  const dim3 grid((unsigned)(a.n_ttiles * a.n_splits)), block(kFusedWG);
   FusedPartial* p0 = reinterpret_cast<FusedPartial*>(ws + off_partials(n_tokens));
-  FusedPartial* p1 = reinterpret_cast<FusedPartial*>(ws + off_partials(n_tokens) + partial_bytes(n_tokens, V));
+  FusedPartial* p1 = reinterpret_cast<FusedPartial*>(ws + off_partials(n_tokens) + partial_bytes(n_tokens, H, V));
 
   a.weight = static_cast<const char*>(w0);
   a.partials = p0;
-  if (out_entropy) hipLaunchKernelGGL(fused_lmhead_kernel<true>, grid, block, 0, stream, a);
-  else hipLaunchKernelGGL(fused_lmhead_kernel<false>, grid, block, 0, stream, a);
+  if (out_entropy) launch_main<true>(a, dma, stream);
+  else launch_main<false>(a, dma, stream);
   if (w1) {
     a.weight = static_cast<const char*>(w1);
     a.partials = p1;
-    hipLaunchKernelGGL(fused_lmhead_kernel<false>, grid, block, 0, stream, a);
+    launch_main<false>(a, dma, stream);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
