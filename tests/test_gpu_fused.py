@@ -140,3 +140,42 @@ def test_fused_rejects_bad_inputs(dev):
         tome_amd.fused_lmhead_logprobs(h, w, t, 0.0)
     with pytest.raises(ValueError):
         tome_amd.fused_lmhead_logprobs(h[:, :60], w[:, :60].contiguous(), t)   # H % 8 != 0
+
+
+@pytest.mark.parametrize("n,H,V", [(200, 256, 5000), (70, 72, 1000), (300, 1024, 20000)])
+def test_fused_argmax(dev, n, H, V):
+    """Greedy id: exact where the top-2 gap exceeds fp32 accumulation noise, lowest index on exact ties."""
+    h, w, t = _inputs(dev, n, H, V, seed=V + n, w_scale=0.1)
+    r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 1.0, want_argmax=True)
+    want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(w), t, 1.0)
+    clear = (want["top1"] - want["top2"]) > 1e-3
+    assert clear.mean() > 0.9
+    got = r.argmax.cpu().numpy()
+    np.testing.assert_array_equal(got[clear], want["argmax"][clear])
+    # near ties: whatever is returned must be within noise of the maximum
+    logits = oracle.lmhead_logits64(bf16_bits_of(h), bf16_bits_of(w))
+    assert (want["top1"] - logits[np.arange(n), got] <= 1e-3).all()
+
+
+def test_fused_argmax_spike_and_ties(dev):
+    n, H, V = 160, 128, 3000
+    rng = np.random.default_rng(12)
+    h = torch.from_numpy(rng.standard_normal((n, H)).astype(np.float32)).to(dev).to(torch.bfloat16)
+    w32 = (rng.standard_normal((V, H)) * 0.05).astype(np.float32)
+    # rows 100, 1500 and 2999 are identical and aligned with every token: a three-way exact tie at the top
+    w32[[100, 1500, 2999]] = 0.0
+    wt = torch.from_numpy(w32).to(dev).to(torch.bfloat16)
+    hb = h.float()
+    big = (hb / hb.norm(dim=-1, keepdim=True)).mean(0)
+    wt[[100, 1500, 2999]] = (big * 50).to(torch.bfloat16)
+    t = torch.zeros(n, dtype=torch.int32, device=dev)
+    r = tome_amd.fused_lmhead_logprobs(h, wt, t, 1.0, want_argmax=True)
+    want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(wt), np.zeros(n, np.int32), 1.0)
+    tied = want["argmax"] == 100
+    assert tied.sum() > 0
+    got = r.argmax.cpu().numpy()
+    assert (got[tied] == 100).all()                  # first of the tied rows, in different vocab tiles
+    clear = (want["top1"] - want["top2"]) > 1e-3
+    np.testing.assert_array_equal(got[clear], want["argmax"][clear])
+    masked = tome_amd.fused_lmhead_logprobs(h, wt, t, 1.0, want_argmax=True, row_valid=torch.zeros(n, dtype=torch.int32, device=dev))
+    assert (masked.argmax.cpu().numpy() == -1).all()

@@ -289,37 +289,50 @@ __global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) 
 
 
 // ===============================================================================================
-// Fast path (H % 64 == 0): 512 lanes, 256 x 256 tile, K slabs DMA'd straight into LDS.
+// Fast path (H % 32 == 0): 512 lanes, 256 x 256 tile, K slabs DMA'd straight into LDS through a
+// four-slab ring.
 //
 //   * 8 waves as 2 (vocab) x 4 (token); the per-wave tile is still 128 vocab x 64 tokens, so
 //     fold_tile / write_partials and the partial layout are shared with the generic kernel.
 //   * global_load_lds_dwordx4: every lane fetches 16 bytes and the wave's 1 KB lands contiguously
 //     in LDS, bypassing registers.  No staging registers are needed, which leaves room to
-//     double-buffer the MFMA fragments (LDS reads of sub-step k+1 fly during the MFMAs of k).
-//   * LDS holds two 64 KB slabs (W 256 rows + hidden 256 rows, 128 bytes per row, no padding).
-//     The slab for step s+1 is requested at the start of step s and waited for at its end: one
-//     barrier per slab, latency hidden behind 32 MFMAs per wave.  Steps run across vocab-tile
-//     boundaries, so the first slab of the next tile streams in during the epilogue.
+//     double-buffer the MFMA fragments.
+//   * What bounds this kernel is the L2 -> LDS fill (64 KB per 256x256x64 MACs and CU): measured
+//     alone, with one slab in flight, it takes as long as the MFMAs.  Hence a ring of four 32 KB
+//     slabs (K = 32 each: W 256 rows + hidden 256 rows, 64 bytes per row) with three requests in
+//     flight.  Step s (one slab = two MFMA sub-steps) runs
+//         reads(s, k1) | MFMA(s, k0) | wait slab s+1, barrier, request slab s+3 |
+//         reads(s+1, k0) | MFMA(s, k1)
+//     The barrier sits mid-step: everybody is then past step s-1, so its slab can be refilled,
+//     and slab s+1 is visible before its first fragments are read, which happens under the
+//     second half of the MFMAs - the MFMA stream has no bubble at step or vocab-tile boundaries.
 //   * Bank conflicts are avoided by an XOR swizzle instead of padding (DMA writes are dense).
 //     The LDS has 64 four-byte banks, so a 16-lane phase of a 128-bit read is conflict-free when
-//     its 16 rows hit 16 different 16-byte bank groups.  Row r covers groups 8*(r&1) .. +7, so
-//     chunk c of row r is stored at chunk position c ^ ((r >> 1) & 7); the lane that DMA-writes
-//     position p of row r fetches global chunk p ^ ((r >> 1) & 7).
+//     its 16 rows hit 16 different 16-byte bank groups.  A 64-byte row r covers groups
+//     4*(r&3) .. +3, so chunk c of row r is stored at chunk position c ^ ((r >> 2) & 3); the
+//     lane that DMA-writes position p of row r fetches global chunk p ^ ((r >> 2) & 3).
 // ===============================================================================================
 constexpr int k2BV = 256, k2BT = 256, k2WG = 512;
-constexpr int k2RowBytes = kBK * 2;                    // 128
-constexpr int k2SlabBytes = (k2BV + k2BT) * k2RowBytes;  // 65536
-constexpr int k2LdsBytes = 2 * k2SlabBytes;
-constexpr int k2LdsTotal = k2LdsBytes;
-constexpr int k2Loads = k2BV * 8 / k2WG;               // DMA instructions per lane per operand per slab (4)
+constexpr int k2BK = 32;
+constexpr int k2RowBytes = k2BK * 2;                     // 64
+constexpr int k2SlabBytes = (k2BV + k2BT) * k2RowBytes;  // 32768
+constexpr int k2Slabs = 4;
+constexpr int k2LdsTotal = k2Slabs * k2SlabBytes;        // 131072
+constexpr int k2Loads = k2BV * (k2RowBytes / 16) / k2WG; // DMA instructions per lane, operand and slab (2)
+constexpr int k2DmaPerSlab = 2 * k2Loads;                // vmcnt units per slab and wave
 
 __device__ __forceinline__ void dma16(const char* gptr, char* lds_wave_base) {
   __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(gptr),
-                                   reinterpret_cast<__attribute__((address_space(3))) uint32_t*>(
-                                       reinterpret_cast<__attribute__((address_space(3))) char*>(
-                                           (__attribute__((address_space(3))) char*)lds_wave_base)),
-                                   16, 0, 0);
+                                   (__attribute__((address_space(3))) uint32_t*)lds_wave_base, 16, 0, 0);
 }
+
+// Wait until at most `slabs` of this wave's slab requests are still in flight.
+__device__ __forceinline__ void wait_slabs(int slabs) {
+  if (slabs >= 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else if (slabs == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+static_assert(k2DmaPerSlab == 4 && kNBV == 4, "wait_slabs and the DMA interleave assume 4 DMA instructions per slab");
 
 template <bool ENT>
 __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
@@ -341,17 +354,17 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   const int wave_v = wave & 1, wave_t = wave >> 1;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  // ---- DMA assignment: instruction j of wave w fills LDS rows (j*8 + w)*8 .. +7 of an operand ----
-  // All address arithmetic is incremental: per-lane pointers advance by one slab (128 bytes) per
-  // step and are rebased at vocab-tile changes, so a step carries no multiplies or divides.
-  const int dr = lane >> 3;                                   // row inside the 8-row group
-  const int dc = (lane & 7) ^ (((wave & 1) << 2) | (dr >> 1));  // global chunk: position ^ ((row >> 1) & 7)
+  // ---- DMA assignment: instruction j of wave w fills LDS rows (j*8 + w)*16 .. +15 of an operand --
+  // All address arithmetic is incremental: per-lane pointers advance by one slab (64 bytes) per
+  // request and are rebased at vocab-tile changes, so a step carries no multiplies or divides.
+  const int dr = lane >> 2;                       // row inside the 16-row group
+  const int dc = (lane & 3) ^ ((dr >> 2) & 3);    // global chunk: position ^ ((row >> 2) & 3)
   const char* pa[k2Loads];  // next W slab to request, per DMA instruction
   const char* pb[k2Loads];  // next hidden slab
   auto point_a = [&](int vt) {  // rows past V (last tile only) read the last row; masked in the epilogue
 #pragma unroll
     for (int j = 0; j < k2Loads; ++j) {
-      int64_t v = (int64_t)vt * k2BV + (j * 8 + wave) * 8 + dr;
+      int64_t v = (int64_t)vt * k2BV + (j * 8 + wave) * 16 + dr;
       v = v < a.V ? v : a.V - 1;
       pa[j] = a.weight + v * a.weight_stride_b + dc * 16;
     }
@@ -359,7 +372,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   point_a(vt0);
 #pragma unroll
   for (int j = 0; j < k2Loads; ++j) {
-    int p = t0 + (j * 8 + wave) * 8 + dr;
+    int p = t0 + (j * 8 + wave) * 16 + dr;
     p = p < n_valid ? p : n_valid - 1;
     const int tok = a.row_index ? a.row_index[p] : p;
     pb[j] = a.hidden + (int64_t)tok * a.hidden_stride_b + dc * 16;
@@ -379,25 +392,25 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   }
 
   // ---- fragment read offsets inside a slab (swizzled) --------------------------------------------
-  const int x7 = (l32 >> 1) & 7;
-  int swz[kBK / 16];
-#pragma unroll
-  for (int ks = 0; ks < kBK / 16; ++ks) swz[ks] = ((ks * 2 + lh) ^ x7) * 16;
+  const int x3 = (l32 >> 2) & 3;
+  const int swz0 = ((0 + lh) ^ x3) * 16, swz1 = ((2 + lh) ^ x3) * 16;
   const int rdA = (wave_v * kWaveV + l32) * k2RowBytes;
   const int rdB = k2BV * k2RowBytes + (wave_t * kWaveT + l32) * k2RowBytes;
 
-  const int nk = a.H / kBK;
-  const int64_t slab_rewind = (int64_t)nk * k2RowBytes;
+  const int nk = a.H / k2BK;
+  const int n_steps = (vt1 - vt0) * nk;
+  const int64_t slab_rewind = (int64_t)(nk - 1) * k2RowBytes;
   int i_kt = 0, i_vt = vt0;  // slab the next `issue` will request
-  int buf = 0;               // LDS slab that request lands in
+  int issued = 0;            // slabs requested so far; request q lands in ring slot q % 4
 
-  auto issue = [&]() {
-    char* dst = smem + buf * k2SlabBytes + wave * 1024;
-#pragma unroll
-    for (int j = 0; j < k2Loads; ++j) dma16(pa[j], dst + j * 8192);
-#pragma unroll
-    for (int j = 0; j < k2Loads; ++j) dma16(pb[j], dst + k2BV * k2RowBytes + j * 8192);
-    buf ^= 1;
+  // One of the four DMA instructions of the next request (0,1: W rows; 2,3: hidden rows).
+  auto issue_piece = [&](int piece) {
+    char* dst = smem + (issued & (k2Slabs - 1)) * k2SlabBytes + wave * 1024;
+    if (piece < k2Loads) dma16(pa[piece], dst + piece * 8192);
+    else dma16(pb[piece - k2Loads], dst + k2BV * k2RowBytes + (piece - k2Loads) * 8192);
+  };
+  auto issue_done = [&]() {
+    ++issued;
     if (++i_kt < nk) {
 #pragma unroll
       for (int j = 0; j < k2Loads; ++j) {
@@ -408,75 +421,87 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
       i_kt = 0;
       ++i_vt;
 #pragma unroll
-      for (int j = 0; j < k2Loads; ++j) pb[j] -= slab_rewind - k2RowBytes;
+      for (int j = 0; j < k2Loads; ++j) pb[j] -= slab_rewind;
       if (i_vt < vt1) point_a(i_vt);
     }
   };
+  auto issue = [&]() {
+#pragma unroll
+    for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
+    issue_done();
+  };
+  auto read_frags = [&](int step, int sw, bf16x8 (&fa)[kNBV], bf16x8 (&fb)[kNBT]) {
+    const char* slab = smem + (step & (k2Slabs - 1)) * k2SlabBytes;
+#pragma unroll
+    for (int i = 0; i < kNBV; ++i)
+      fa[i] = *reinterpret_cast<const bf16x8*>(slab + rdA + i * 32 * k2RowBytes + sw);
+#pragma unroll
+    for (int j = 0; j < kNBT; ++j)
+      fb[j] = *reinterpret_cast<const bf16x8*>(slab + rdB + j * 32 * k2RowBytes + sw);
+  };
 
-  issue();
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  for (int q = 0; q < 3 && q < n_steps; ++q) issue();
+  wait_slabs(issued - 1);
   __syncthreads();
 
-  int cur = 0;
+  bf16x8 fa0[kNBV], fb0[kNBT], fa1[kNBV], fb1[kNBT];
+  read_frags(0, swz0, fa0, fb0);
+
+  f32x16 acc[kNBV][kNBT];
+#pragma unroll
+  for (int i = 0; i < kNBV; ++i)
+#pragma unroll
+    for (int j = 0; j < kNBT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  int step = 0;
   for (int vt = vt0; vt < vt1; ++vt) {
-    f32x16 acc[kNBV][kNBT];
+    for (int kt = 0; kt < nk; ++kt, ++step) {
+      // Scheduling fences pin the software pipeline; left alone, the scheduler sinks every LDS
+      // read next to its use and serialises read latency with the MFMAs.
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(step, swz1, fa1, fb1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < kNBV; ++i)
+#pragma unroll
+        for (int j = 0; j < kNBT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0[i], fb0[j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // Slab step+1 has landed for this wave; after the (fence-less) barrier it has for everyone,
+      // and everyone is past step-1, whose ring slot the next request overwrites.
+      wait_slabs(issued - (step + 2));
+      __builtin_amdgcn_s_barrier();
+      const bool more = issued < n_steps;
+      __builtin_amdgcn_sched_barrier(0);
+      // Unconditional (after the last step it re-reads a stale slot, unused): a branch here
+      // makes the wait-count insertion treat these reads as possibly absent and drain them.
+      read_frags(step + 1, swz0, fa0, fb0);
+      __builtin_amdgcn_sched_barrier(0);
+      // The next request is spread over the MFMAs (one DMA instruction per two MFMAs): all eight
+      // waves leave the barrier together, and a burst of 32 KB requests would back up the
+      // address queue and stall the in-order waves in front of their MFMAs.
+#pragma unroll
+      for (int i = 0; i < kNBV; ++i) {
+#pragma unroll
+        for (int j = 0; j < kNBT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1[i], fb1[j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) issue_piece(i);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (more) issue_done();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const int v0 = vt * k2BV;
+    fold_tile<ENT>(acc, st, tx, tgt, v0 + wave_v * kWaveV, lh, v0 + k2BV > a.V, a.V, a.scale);
 #pragma unroll
     for (int i = 0; i < kNBV; ++i)
 #pragma unroll
       for (int j = 0; j < kNBT; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-    for (int kt = 0; kt < nk; ++kt) {
-      // Request the next slab (possibly the first slab of the next vocab tile, which then
-      // streams in during the epilogue) before touching the current one.
-      if (i_vt < vt1) issue();
-
-      const char* slab = smem + cur * k2SlabBytes;
-      bf16x8 fa[2][kNBV], fb[2][kNBT];
-#pragma unroll
-      for (int i = 0; i < kNBV; ++i)
-        fa[0][i] = *reinterpret_cast<const bf16x8*>(slab + rdA + i * 32 * k2RowBytes + swz[0]);
-#pragma unroll
-      for (int j = 0; j < kNBT; ++j)
-        fb[0][j] = *reinterpret_cast<const bf16x8*>(slab + rdB + j * 32 * k2RowBytes + swz[0]);
-#pragma unroll
-      for (int ks = 0; ks < kBK / 16; ++ks) {
-        const int c = ks & 1, n = c ^ 1;
-        // Scheduling fences pin the software pipeline: the LDS reads of sub-step ks+1 are issued
-        // before the MFMAs of sub-step ks, which then cover their latency.  Left alone, the
-        // scheduler sinks every read next to its use and reuses one fragment register set.
-        __builtin_amdgcn_sched_barrier(0);
-        if (ks + 1 < kBK / 16) {
-#pragma unroll
-          for (int i = 0; i < kNBV; ++i)
-            fa[n][i] = *reinterpret_cast<const bf16x8*>(slab + rdA + i * 32 * k2RowBytes + swz[ks + 1]);
-#pragma unroll
-          for (int j = 0; j < kNBT; ++j)
-            fb[n][j] = *reinterpret_cast<const bf16x8*>(slab + rdB + j * 32 * k2RowBytes + swz[ks + 1]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < kNBV; ++i)
-#pragma unroll
-          for (int j = 0; j < kNBT; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[c][i], fb[c][j], acc[i][j], 0, 0, 0);
-      }
-
-      if (kt == nk - 1) {
-        const int v0 = vt * k2BV;
-#ifndef TOME_EXP_NOFOLD
-        fold_tile<ENT>(acc, st, tx, tgt, v0 + wave_v * kWaveV, lh, v0 + k2BV > a.V, a.V, a.scale);
-#else
-        for (int i = 0; i < kNBV; ++i) for (int j = 0; j < kNBT; ++j) st[j].s += acc[i][j][0] + v0;
-#endif
-      }
-      cur ^= 1;
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next slab has landed
-      // Bare barrier (no fence): LDS reads of the current slab were consumed by the MFMAs above and
-      // the DMA writes are covered by the explicit wait, so nothing else needs draining.
-      __builtin_amdgcn_s_barrier();
-    }
   }
 
   write_partials(st, tx, a.partials, t0 + wave_t * kWaveT, n_valid, split * kPartsPerSplit + wave_v,
@@ -541,10 +566,57 @@ struct CombineArgs {
   float* out_entropy;
   float* out_ref_lp;
   float* out_k3;
+  int32_t* out_argmax;
+  const char* hidden;  // only read when out_argmax is set
+  const char* weight;
+  uint32_t hidden_stride_b;
+  uint32_t weight_stride_b;
+  int H;
+  int V;
   int n_tokens;
   int n_parts;
   float scale;
 };
+
+// Greedy token id of one token.  The sweep only records WHICH 32-row vocab block held the
+// row maximum (first block on ties); the 32 logits of that block are recomputed here as
+// fp32 dot products (lanes l and l+32 take the two halves of K) and the first maximum wins.
+__device__ __forceinline__ int argmax_in_block(const CombineArgs& a, int tok, int block0, int lane) {
+  if (block0 < 0 || block0 >= a.V) return 0;  // nothing above the floor was seen
+  const int row = block0 + (lane & 31), half = lane >> 5;
+  float d = -INFINITY;
+  if (row < a.V) {
+    const u32x4* w = reinterpret_cast<const u32x4*>(a.weight + (int64_t)row * a.weight_stride_b);
+    const u32x4* h = reinterpret_cast<const u32x4*>(a.hidden + (int64_t)tok * a.hidden_stride_b);
+    const int n_chunks = a.H / 8, mid = (n_chunks + 1) / 2;
+    float acc = 0.f;
+    for (int c = half ? mid : 0; c < (half ? n_chunks : mid); ++c) {
+      const u32x4 wv = w[c], hv = h[c];
+      acc = fmaf(bf16_lo(wv.x), bf16_lo(hv.x), acc);
+      acc = fmaf(bf16_hi(wv.x), bf16_hi(hv.x), acc);
+      acc = fmaf(bf16_lo(wv.y), bf16_lo(hv.y), acc);
+      acc = fmaf(bf16_hi(wv.y), bf16_hi(hv.y), acc);
+      acc = fmaf(bf16_lo(wv.z), bf16_lo(hv.z), acc);
+      acc = fmaf(bf16_hi(wv.z), bf16_hi(hv.z), acc);
+      acc = fmaf(bf16_lo(wv.w), bf16_lo(hv.w), acc);
+      acc = fmaf(bf16_hi(wv.w), bf16_hi(hv.w), acc);
+    }
+    d = acc;
+  }
+  const float other = __shfl_xor(d, 32, 64);
+  d = row < a.V ? d + other : -INFINITY;  // both halves now hold the full dot product
+  int idx = lane & 31;
+#pragma unroll
+  for (int off = 16; off > 0; off >>= 1) {
+    const float od = __shfl_xor(d, off, 64);
+    const int oi = __shfl_xor(idx, off, 64);
+    if (od > d || (od == d && oi < idx)) {
+      d = od;
+      idx = oi;
+    }
+  }
+  return block0 + idx;
+}
 
 __device__ __forceinline__ void combine_one(const FusedPartial* parts, int n_parts, int lane, float scale,
                                             RowStat& st, float& tx) {
@@ -582,7 +654,10 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
     const float mr = sr.mx * a.scale;
     ref_lp = txr == -INFINITY ? __builtin_nanf("") : (fmaf(txr, a.scale, -mr) - fast_log2(sr.s)) * kLn2;
   }
+  int amax = 0;
+  if (a.out_argmax) amax = argmax_in_block(a, tok, st.bi == 0x7fffffff ? -1 : st.bi, lane);
   if (lane != 0) return;
+  if (a.out_argmax) a.out_argmax[tok] = amax;
   if (a.out_lp) a.out_lp[tok] = lp;
   if (a.out_lse) a.out_lse[tok] = (m + log2s) * kLn2;
   if (a.out_entropy) a.out_entropy[tok] = (m + log2s - st.w / st.s) * kLn2;
@@ -594,9 +669,9 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
 }
 
 // ---- host side -----------------------------------------------------------------------------------
-// The DMA kernel needs whole 64-wide K slabs and pays for 256-token tiles; short batches and
+// The DMA kernel needs whole 32-wide K slabs and pays for 256-token tiles; short batches and
 // ragged H go to the generic kernel.
-static bool use_dma_kernel(int64_t n_tokens, int64_t H) { return H % kBK == 0 && n_tokens > kBT; }
+static bool use_dma_kernel(int64_t n_tokens, int64_t H) { return H % k2BK == 0 && n_tokens > kBT; }
 
 static int fused_splits(int64_t n_tokens, int64_t H, int64_t V) {
   const bool dma = use_dma_kernel(n_tokens, H);
@@ -700,11 +775,17 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w
   c.out_entropy = out_entropy;
   c.out_ref_lp = out_ref_lp;
   c.out_k3 = out_k3;
+  c.out_argmax = out_argmax;
+  c.hidden = a.hidden;
+  c.weight = static_cast<const char*>(w0);
+  c.hidden_stride_b = a.hidden_stride_b;
+  c.weight_stride_b = a.weight_stride_b;
+  c.H = a.H;
+  c.V = a.V;
   c.n_tokens = (int)n_tokens;
   c.n_parts = a.n_splits * kPartsPerSplit;
   c.scale = a.scale;
   hipLaunchKernelGGL(fused_combine_kernel, dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, stream, c);
-  (void)out_argmax;
   return hipGetLastError();
 }
 

@@ -208,12 +208,14 @@ def _check_fused_inputs(hidden: torch.Tensor, *weights: torch.Tensor):
 
 def fused_lmhead_logprobs(hidden: torch.Tensor, weight: torch.Tensor, targets, temperature: float = 1.0,
                           lengths=None, *, row_valid=None, want_lse: bool = False,
-                          want_entropy: bool = False) -> TokenLogprobs:
+                          want_entropy: bool = False, want_argmax: bool = False) -> TokenLogprobs:
     """Log-probs of ``targets`` under softmax((hidden @ weight.T) / temperature) without the logits.
 
     ``hidden`` [..., H] bf16 (already through the final norm, mlx-impl/model.py:536),
     ``weight`` [V, H] bf16 (the tied embedding matrix, model.py:538).  bf16 products are
     accumulated in fp32; unlike the reference the logits are not rounded to bf16.
+    ``want_argmax`` adds the greedy token id (first maximum, as ``int(mx.argmax(logits))`` at
+    mlx-impl/node.py:897); logits closer than fp32 accumulation noise may swap.
     """
     lib = _lib.load_library()
     dev, lead, h2, (w,) = _check_fused_inputs(hidden, weight)
@@ -226,16 +228,17 @@ def fused_lmhead_logprobs(hidden: torch.Tensor, weight: torch.Tensor, targets, t
         lp = torch.empty(n, dtype=torch.float32, device=dev)
         lse = torch.empty(n, dtype=torch.float32, device=dev) if want_lse else None
         ent = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
+        amax = torch.empty(n, dtype=torch.int32, device=dev) if want_argmax else None
         ws_bytes = lib.tome_fused_lmhead_logprob_workspace(n, H, V)
         ws = _workspace(ws_bytes, dev)
         _lib.check(lib.tome_fused_lmhead_logprob(h2.data_ptr(), w.data_ptr(), n, H, V,
                                                  h2.stride(0) if n > 1 else H, w.stride(0),
                                                  tg.data_ptr(), _ptr(rv), temperature, lp.data_ptr(), _ptr(lse),
-                                                 _ptr(ent), None, _ptr(ws), ws_bytes, _stream(dev)))
+                                                 _ptr(ent), _ptr(amax), _ptr(ws), ws_bytes, _stream(dev)))
 
     def _shaped(t):
         return None if t is None else t.reshape(lead)
-    return TokenLogprobs(_shaped(lp), _shaped(lse), _shaped(ent), None)
+    return TokenLogprobs(_shaped(lp), _shaped(lse), _shaped(ent), _shaped(amax))
 
 
 def grpo_dual_logprobs(hidden: torch.Tensor, w_policy: torch.Tensor, w_ref: torch.Tensor, targets,
