@@ -25,6 +25,12 @@ if ROOT not in sys.path:
 V = 151936
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+# HBM-side bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE counter passes, each scaled by the same
+# counter's reading for a plain 2^30-byte copy (profiles/hbm_traffic_counters.txt).  The masked figure
+# belongs to the seeded lengths of make_config2 (2356 valid rows).
+TRAFFIC_ROW_MASKED = 716.6e6 + 0.13e6
+TRAFFIC_ROW_ALL = 1245.4e6 + 0.13e6
+TRAFFIC_FUSED_CFG3 = 2805e6 + 4.4e6
 
 
 def log(*a):
@@ -69,7 +75,7 @@ def time_steps(fn, steps, warmup):
     return start.elapsed_time(stop) / steps, wall_ms
 
 
-def bench_row(dev, steps, warmup):
+def bench_row(dev, steps, warmup, variant="both"):
     import torch
     import tome_amd
     from tome_amd import _lib
@@ -98,8 +104,8 @@ def bench_row(dev, steps, warmup):
     assert torch.isfinite(got).all() and (got <= 1e-5).all()
     assert (got[valid == 0] == 0).all()
 
-    ms_mask, wall_mask = time_steps(lambda: step(True), steps, warmup)
-    ms_all, wall_all = time_steps(lambda: step(False), steps, warmup)
+    ms_mask, wall_mask = time_steps(lambda: step(True), steps, warmup) if variant in ("both", "mask") else (float("nan"),) * 2
+    ms_all, wall_all = time_steps(lambda: step(False), steps, warmup) if variant in ("both", "all") else (float("nan"),) * 2
     bytes_mask = n_valid * V * 2
     bytes_all = rows * V * 2
     out = {
@@ -185,6 +191,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", choices=["row", "fused"], default=None)
+    ap.add_argument("--row-variant", choices=["both", "mask", "all"], default="both",
+                    help="time config 2 with its padding mask, without it, or both (profiling runs pick one)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy, so a counter run can scale FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this path is measured on ONE GPU (rows are independent; more GPUs would each run "
@@ -201,7 +211,14 @@ def main():
     torch.cuda.set_device(dev)
     log("device:", torch.cuda.get_device_name(dev))
 
-    row = bench_row(dev, args.steps, args.warmup) if args.only in (None, "row") else None
+    if args.calibrate_copy:   # known traffic: 2^30 bytes read + 2^30 bytes written per copy
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    row = bench_row(dev, args.steps, args.warmup, args.row_variant) if args.only in (None, "row") else None
     fused = bench_fused(dev, max(5, args.steps // 2), max(2, args.warmup // 2)) if args.only in (None, "fused") else None
     cpu = None if args.no_cpu else cpu_baseline()
 
@@ -212,6 +229,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "data": "synthetic", "dtype": "f32",
     }
+    if row is not None and args.row_variant == "all":
+        row["ms_mask"], row["gbs_mask"], row["bytes_mask"], row["n_valid"] = (row["ms_all"], row["gbs_all"],
+                                                                              row["bytes_all"], row["rows"])
     if row is not None:
         line.update({
             "value": row["n_valid"] / (row["ms_mask"] * 1e-3),
@@ -220,21 +240,27 @@ def main():
                                    "padding mask lengths~U[64,512], fp32 out",
                        "rows": row["rows"], "valid_rows": row["n_valid"], "vocab": V, "temperature": 1.0},
             "roofline": {"bound": "hbm", "achieved": row["gbs_mask"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": row["gbs_mask"] / HBM_PEAK_GBS, "traffic": None,
+                         "frac": row["gbs_mask"] / HBM_PEAK_GBS,
+                         "traffic": TRAFFIC_ROW_ALL if args.row_variant == "all" else TRAFFIC_ROW_MASKED,
                          "kernel": "row_logprob_kernel<bf16>", "bytes_per_launch": row["bytes_mask"]},
-            "all_rows": {"value": row["rows"] / (row["ms_all"] * 1e-3), "ms_per_step": row["ms_all"],
-                         "roofline": {"bound": "hbm", "achieved": row["gbs_all"], "peak": HBM_PEAK_GBS,
-                                      "unit": "GB/s", "frac": row["gbs_all"] / HBM_PEAK_GBS, "traffic": None,
-                                      "bytes_per_launch": row["bytes_all"]}},
         })
+        if args.row_variant == "all":
+            line["config"]["workload"] = line["config"]["workload"].replace(
+                "padding mask lengths~U[64,512]", "padding mask NOT applied (all 4096 rows read)")
+        if args.row_variant == "both":
+            line["all_rows"] = {"value": row["rows"] / (row["ms_all"] * 1e-3), "ms_per_step": row["ms_all"],
+                                "config": {"workload": "config 2 without the padding mask: all 4096 rows read"},
+                                "roofline": {"bound": "hbm", "achieved": row["gbs_all"], "peak": HBM_PEAK_GBS,
+                                             "unit": "GB/s", "frac": row["gbs_all"] / HBM_PEAK_GBS, "traffic": TRAFFIC_ROW_ALL,
+                                             "bytes_per_launch": row["bytes_all"]}}
     if fused is not None:
         f = {"value": fused["tokens"] / (fused["ms"] * 1e-3), "unit": "token-logprobs/s", "ms_per_step": fused["ms"],
              "dtype": "bf16 x bf16 -> f32",
              "config": {"workload": "config 3: fused lm_head + log-softmax, hidden [4096,1024] x W [151936,1024] bf16",
                         "tokens": fused["tokens"], "hidden": fused["H"], "vocab": V},
              "roofline": {"bound": "mfma", "achieved": fused["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
-                          "unit": "TFLOP/s", "frac": fused["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
-                          "kernel": "fused_lmhead_kernel", "flop_per_launch": fused["flop"]}}
+                          "unit": "TFLOP/s", "frac": fused["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": TRAFFIC_FUSED_CFG3,
+                          "kernel": "fused_lmhead_dma_kernel", "flop_per_launch": fused["flop"]}}
         if row is None:
             line.update({"value": f["value"], "ms_per_step": f["ms_per_step"], "config": f["config"],
                          "roofline": f["roofline"], "dtype": "f32"})
