@@ -187,8 +187,8 @@ def cpu_baseline(sample_rows=256, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", choices=["row", "fused"], default=None)
     ap.add_argument("--row-variant", choices=["both", "mask", "all"], default="both",
@@ -219,6 +219,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     row = bench_row(dev, args.steps, args.warmup, args.row_variant) if args.only in (None, "row") else None
+    # the fused step is ~10x longer than a row step: half the launches keep the run short; the clocks
+    # still settle (a few tens of milliseconds of back-to-back launches are needed for that)
     fused = bench_fused(dev, max(5, args.steps // 2), max(2, args.warmup // 2)) if args.only in (None, "fused") else None
     cpu = None if args.no_cpu else cpu_baseline()
 

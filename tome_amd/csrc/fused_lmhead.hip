@@ -59,10 +59,26 @@ struct FusedArgs {
   int H;
   int V;
   int n_vtiles;
-  int n_splits;
-  int n_ttiles;
+  int slots;                 // workgroups that fit the chip at once (the schedule aims at one round)
   float scale;               // log2(e) / temperature
 };
+
+// Work decomposition, computed on the DEVICE from the number of valid tokens (known only there when a
+// mask is given): token tiles x vocab splits, with just enough splits to fill `slots` workgroups.
+// Every kernel of a launch derives the same numbers from the same inputs.
+struct FusedSchedule {
+  int n_ttiles, n_splits, n_wg;
+};
+__host__ __device__ inline FusedSchedule fused_schedule(int n_valid, int bt, int slots, int n_vtiles) {
+  FusedSchedule s;
+  s.n_ttiles = (n_valid + bt - 1) / bt;
+  if (s.n_ttiles < 1) s.n_ttiles = 1;
+  s.n_splits = slots / s.n_ttiles;  // rounded down: one workgroup too many would cost a whole extra round
+  if (s.n_splits > n_vtiles) s.n_splits = n_vtiles;
+  if (s.n_splits < 1) s.n_splits = 1;
+  s.n_wg = s.n_ttiles * s.n_splits;
+  return s;
+}
 
 // Raw buffer descriptors: 16-byte loads addressed by a 32-bit per-lane byte offset plus a
 // uniform (scalar) offset.  A per-lane offset at or past num_bytes reads as zero, which is how
@@ -174,19 +190,19 @@ __global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) 
   char* ldsA = lds;
   char* ldsB = lds + kBV * kPitch;
 
+  const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
+  const FusedSchedule sch = fused_schedule(n_valid, kBT, a.slots, a.n_vtiles);
+  int bid = blockIdx.x;
+  if (n_valid <= 0 || bid >= sch.n_wg) return;  // the grid is sized for the worst case over n_valid
   // XCD-aware remap: hardware deals consecutive workgroup ids round-robin over the 8 XCDs;
   // give each XCD a contiguous block of logical ids (= a few token tiles x all splits) so the
   // hidden tiles it touches stay in its own L2.
-  int bid = blockIdx.x;
-  const int nwg = gridDim.x;
-  if ((nwg & 7) == 0) bid = (bid & 7) * (nwg >> 3) + (bid >> 3);
-  const int ttile = bid / a.n_splits;
-  const int split = bid % a.n_splits;
-  const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
+  if ((sch.n_wg & 7) == 0) bid = (bid & 7) * (sch.n_wg >> 3) + (bid >> 3);
+  const int ttile = bid / sch.n_splits;
+  const int split = bid % sch.n_splits;
   const int t0 = ttile * kBT;
-  if (t0 >= n_valid) return;
-  const int vt0 = (int)((int64_t)split * a.n_vtiles / a.n_splits);
-  const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / a.n_splits);
+  const int vt0 = (int)((int64_t)split * a.n_vtiles / sch.n_splits);
+  const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / sch.n_splits);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wave_v = wave & 1, wave_t = wave >> 1;
@@ -284,7 +300,7 @@ __global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) 
   }
 
   write_partials(st, tx, a.partials, t0 + wave_t * kWaveT, n_valid, split * kPartsPerSplit + wave_v,
-                 a.n_splits * kPartsPerSplit, l32, lh, a.scale);
+                 sch.n_splits * kPartsPerSplit, l32, lh, a.scale);
 }
 
 
@@ -338,17 +354,16 @@ template <bool ENT>
 __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  int bid = blockIdx.x;
-  const int nwg = gridDim.x;
-  if ((nwg & 7) == 0) bid = (bid & 7) * (nwg >> 3) + (bid >> 3);  // contiguous logical ids per XCD
-  const int ttile = bid / a.n_splits;
-  const int split = bid % a.n_splits;
   const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
+  const FusedSchedule sch = fused_schedule(n_valid, k2BT, a.slots, a.n_vtiles);
+  int bid = blockIdx.x;
+  if (n_valid <= 0 || bid >= sch.n_wg) return;  // the grid is sized for the worst case over n_valid
+  if ((sch.n_wg & 7) == 0) bid = (bid & 7) * (sch.n_wg >> 3) + (bid >> 3);  // contiguous logical ids per XCD
+  const int ttile = bid / sch.n_splits;
+  const int split = bid % sch.n_splits;
   const int t0 = ttile * k2BT;
-  if (t0 >= n_valid) return;
-  const int vt0 = (int)((int64_t)split * a.n_vtiles / a.n_splits);
-  const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / a.n_splits);
-  if (vt0 >= vt1) return;
+  const int vt0 = (int)((int64_t)split * a.n_vtiles / sch.n_splits);
+  const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / sch.n_splits);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wave_v = wave & 1, wave_t = wave >> 1;
@@ -505,7 +520,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   }
 
   write_partials(st, tx, a.partials, t0 + wave_t * kWaveT, n_valid, split * kPartsPerSplit + wave_v,
-                 a.n_splits * kPartsPerSplit, l32, lh, a.scale);
+                 sch.n_splits * kPartsPerSplit, l32, lh, a.scale);
 }
 
 // ---- compaction of valid rows ----------------------------------------------------------------
@@ -574,7 +589,7 @@ struct CombineArgs {
   int H;
   int V;
   int n_tokens;
-  int n_parts;
+  int bt, slots, n_vtiles;  // inputs of fused_schedule, to find the number of parts per token
   float scale;
 };
 
@@ -639,9 +654,10 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
   const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
   if (p >= n_valid) return;
   const int tok = a.row_index ? a.row_index[p] : p;
+  const int n_parts = fused_schedule(n_valid, a.bt, a.slots, a.n_vtiles).n_splits * kPartsPerSplit;
   RowStat st;
   float tx;
-  combine_one(a.partials + (int64_t)p * a.n_parts, a.n_parts, lane, a.scale, st, tx);
+  combine_one(a.partials + (int64_t)p * n_parts, n_parts, lane, a.scale, st, tx);
   const float m = st.mx * a.scale;
   const float log2s = fast_log2(st.s);
   // tx stays -inf only when the target id was outside [0, V).
@@ -650,7 +666,7 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
   if (a.partials_ref) {
     RowStat sr;
     float txr;
-    combine_one(a.partials_ref + (int64_t)p * a.n_parts, a.n_parts, lane, a.scale, sr, txr);
+    combine_one(a.partials_ref + (int64_t)p * n_parts, n_parts, lane, a.scale, sr, txr);
     const float mr = sr.mx * a.scale;
     ref_lp = txr == -INFINITY ? __builtin_nanf("") : (fmaf(txr, a.scale, -mr) - fast_log2(sr.s)) * kLn2;
   }
@@ -673,23 +689,37 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
 // ragged H go to the generic kernel.
 static bool use_dma_kernel(int64_t n_tokens, int64_t H) { return H % k2BK == 0 && n_tokens > kBT; }
 
-static int fused_splits(int64_t n_tokens, int64_t H, int64_t V) {
-  const bool dma = use_dma_kernel(n_tokens, H);
-  const int64_t bt = dma ? k2BT : kBT, bv = dma ? k2BV : kBV;
-  const int64_t slots = dma ? 256 : 512;  // resident workgroups on 256 CUs: 1 per CU (128 KB LDS) or 2
-  const int64_t n_ttiles = (n_tokens + bt - 1) / bt;
-  const int64_t n_vtiles = (V + bv - 1) / bv;
-  int64_t s = (slots + n_ttiles - 1) / n_ttiles;
-  if (s > n_vtiles) s = n_vtiles;
-  if (s < 1) s = 1;
-  return (int)s;
+struct FusedPlan {
+  bool dma;
+  int bt, bv, slots, n_vtiles;
+  int grid;            // workgroups to launch: the most any number of valid tokens can ask for
+  size_t max_records;  // partial records any number of valid tokens can produce
+};
+
+static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
+  FusedPlan p;
+  p.dma = use_dma_kernel(n_tokens, H);
+  p.bt = p.dma ? k2BT : kBT;
+  p.bv = p.dma ? k2BV : kBV;
+  p.slots = p.dma ? 256 : 512;  // resident workgroups on 256 CUs: 1 per CU (128 KB LDS) or 2
+  p.n_vtiles = (int)((V + p.bv - 1) / p.bv);
+  p.grid = 0;
+  p.max_records = 0;
+  const int tt_max = (int)((n_tokens + p.bt - 1) / p.bt);
+  for (int tt = 1; tt <= tt_max; ++tt) {  // the schedule depends on n_valid only through its tile count
+    const FusedSchedule s = fused_schedule(tt * p.bt, p.bt, p.slots, p.n_vtiles);
+    if (s.n_wg > p.grid) p.grid = s.n_wg;
+    const size_t rec = (size_t)tt * p.bt * s.n_splits * kPartsPerSplit;
+    if (rec > p.max_records) p.max_records = rec;
+  }
+  return p;
 }
 
 // Layout: [n_valid: 256 B][row_index: n_tokens int32, 256-aligned][partials per weight set].
 static size_t off_index() { return 256; }
 static size_t off_partials(int64_t n_tokens) { return 256 + (((size_t)n_tokens * 4 + 255) & ~(size_t)255); }
 static size_t partial_bytes(int64_t n_tokens, int64_t H, int64_t V) {
-  return (size_t)n_tokens * (size_t)fused_splits(n_tokens, H, V) * kPartsPerSplit * sizeof(FusedPartial);
+  return fused_plan(n_tokens, H, V).max_records * sizeof(FusedPartial);
 }
 
 size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights) {
@@ -697,7 +727,7 @@ size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weigh
 }
 
 template <bool ENT>
-static void launch_main(const FusedArgs& a, bool dma, hipStream_t stream) {
+static void launch_main(const FusedArgs& a, bool dma, int grid, hipStream_t stream) {
   if (dma) {
     static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
     if (!attr_set) {
@@ -705,10 +735,10 @@ static void launch_main(const FusedArgs& a, bool dma, hipStream_t stream) {
                                 hipFuncAttributeMaxDynamicSharedMemorySize, k2LdsTotal);
       attr_set = true;
     }
-    hipLaunchKernelGGL(fused_lmhead_dma_kernel<ENT>, dim3((unsigned)(a.n_ttiles * a.n_splits)), dim3(k2WG),
+    hipLaunchKernelGGL(fused_lmhead_dma_kernel<ENT>, dim3((unsigned)grid), dim3(k2WG),
                        k2LdsTotal, stream, a);
   } else {
-    hipLaunchKernelGGL(fused_lmhead_kernel<ENT>, dim3((unsigned)(a.n_ttiles * a.n_splits)), dim3(kFusedWG), 0,
+    hipLaunchKernelGGL(fused_lmhead_kernel<ENT>, dim3((unsigned)grid), dim3(kFusedWG), 0,
                        stream, a);
   }
 }
@@ -744,23 +774,22 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w
   a.n_tokens = (int)n_tokens;
   a.H = (int)H;
   a.V = (int)V;
-  const bool dma = use_dma_kernel(n_tokens, H);
-  const int64_t bt = dma ? k2BT : kBT, bv = dma ? k2BV : kBV;
-  a.n_vtiles = (int)((V + bv - 1) / bv);
-  a.n_splits = fused_splits(n_tokens, H, V);
-  a.n_ttiles = (int)((n_tokens + bt - 1) / bt);
+  const FusedPlan plan = fused_plan(n_tokens, H, V);
+  const bool dma = plan.dma;
+  a.n_vtiles = plan.n_vtiles;
+  a.slots = plan.slots;
   a.scale = kLog2e / temperature;
   FusedPartial* p0 = reinterpret_cast<FusedPartial*>(ws + off_partials(n_tokens));
   FusedPartial* p1 = reinterpret_cast<FusedPartial*>(ws + off_partials(n_tokens) + partial_bytes(n_tokens, H, V));
 
   a.weight = static_cast<const char*>(w0);
   a.partials = p0;
-  if (out_entropy) launch_main<true>(a, dma, stream);
-  else launch_main<false>(a, dma, stream);
+  if (out_entropy) launch_main<true>(a, dma, plan.grid, stream);
+  else launch_main<false>(a, dma, plan.grid, stream);
   if (w1) {
     a.weight = static_cast<const char*>(w1);
     a.partials = p1;
-    launch_main<false>(a, dma, stream);
+    launch_main<false>(a, dma, plan.grid, stream);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
@@ -783,7 +812,9 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w
   c.H = a.H;
   c.V = a.V;
   c.n_tokens = (int)n_tokens;
-  c.n_parts = a.n_splits * kPartsPerSplit;
+  c.bt = plan.bt;
+  c.slots = plan.slots;
+  c.n_vtiles = plan.n_vtiles;
   c.scale = a.scale;
   hipLaunchKernelGGL(fused_combine_kernel, dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, stream, c);
   return hipGetLastError();
