@@ -179,3 +179,23 @@ def test_fused_argmax_spike_and_ties(dev):
     np.testing.assert_array_equal(got[clear], want["argmax"][clear])
     masked = tome_amd.fused_lmhead_logprobs(h, wt, t, 1.0, want_argmax=True, row_valid=torch.zeros(n, dtype=torch.int32, device=dev))
     assert (masked.argmax.cpu().numpy() == -1).all()
+
+
+@pytest.mark.parametrize("kind", ["generic", "dma", "wide"])
+def test_fused_every_kernel_path(dev, kind, monkeypatch):
+    """The three GEMM kernels behind tome_fused_lmhead_logprob (generic / LDS-DMA ring / wide) are picked
+    by shape; the TOME_FUSED_KERNEL tuning knob forces each of them onto the same problem."""
+    monkeypatch.setenv("TOME_FUSED_KERNEL", kind)
+    n, H, V = 700, 256, 9000          # 3 token tiles of 256 (one ragged), partial last vocab tile, H % 128 == 0
+    h, w, t = _inputs(dev, n, H, V, seed=31, w_scale=0.1)
+    valid = (np.random.default_rng(1).random(n) < 0.7).astype(np.int32)
+    r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 0.8, want_lse=True, want_entropy=True,
+                                       want_argmax=True, row_valid=torch.from_numpy(valid).to(dev))
+    want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(w), t, 0.8)
+    m = valid.astype(bool)
+    np.testing.assert_allclose(r.lp.cpu().numpy()[m], want["lp"][m], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.lse.cpu().numpy()[m], want["lse"][m], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.entropy.cpu().numpy()[m], want["entropy"][m], atol=TOL, rtol=0)
+    clear = m & ((want["top1"] - want["top2"]) > 1e-3)
+    np.testing.assert_array_equal(r.argmax.cpu().numpy()[clear], want["argmax"][clear])
+    assert (r.lp.cpu().numpy()[~m] == 0).all() and (r.argmax.cpu().numpy()[~m] == -1).all()

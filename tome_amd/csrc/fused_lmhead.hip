@@ -22,6 +22,8 @@
 //   * Masked tokens are compacted first (compact_rows_kernel); token tiles are built from
 //     the compacted index list, so masked rows cost no FLOPs and no HBM traffic.
 #include "common.hpp"
+#include <cstdlib>
+#include <type_traits>
 
 namespace tome {
 
@@ -91,39 +93,42 @@ __device__ __forceinline__ u32x4 ld16(__amdgpu_buffer_rsrc_t r, uint32_t lane_of
 }
 
 
-// Fold one wave tile of logits (kNBV x kNBT blocks of 32x32 accumulators) into the per-token
+// Fold one wave tile of logits (NBV x NBT blocks of 32x32 accumulators) into the per-token
 // running states.  Accumulator element e of block i holds vocab row
 //   vw0 + i*32 + 8*(e/4) + 4*lh + e%4        (vw0 = first vocab row of this wave's tile)
 // for the token this lane owns in block column j.
-template <bool ENT>
-__device__ __forceinline__ void fold_tile(f32x16 (&acc)[kNBV][kNBT], RowStat (&st)[kNBT], float (&tx)[kNBT],
-                                          const int (&tgt)[kNBT], int vw0, int lh, bool partial_tile, int V,
+template <bool ENT, int NBV, int NBT>
+__device__ __forceinline__ void fold_tile(f32x16 (&acc)[NBV][NBT], RowStat (&st)[NBT], float (&tx)[NBT],
+                                          const int (&tgt)[NBT], int vw0, int lh, bool partial_tile, int V,
                                           float scale) {
   if (partial_tile) {  // last vocab tile: rows past V do not exist
 #pragma unroll
-    for (int i = 0; i < kNBV; ++i)
+    for (int i = 0; i < NBV; ++i)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const bool dead = vw0 + 4 * lh + i * 32 + 8 * (e / 4) + (e % 4) >= V;
 #pragma unroll
-        for (int j = 0; j < kNBT; ++j) acc[i][j][e] = dead ? -INFINITY : acc[i][j][e];
+        for (int j = 0; j < NBT; ++j) acc[i][j][e] = dead ? -INFINITY : acc[i][j][e];
       }
   }
 #pragma unroll
-  for (int j = 0; j < kNBT; ++j) {
+  for (int j = 0; j < NBT; ++j) {
+    // One scheduling region per token block: otherwise all accumulator reads of all blocks are
+    // hoisted to the top and the register file overflows.
+    __builtin_amdgcn_sched_barrier(0);
     // Target capture: rare (one tile in V/256 per token), so behind a wave-uniform test.
     const int rel = tgt[j] - vw0;
-    const bool mine = tgt[j] >= 0 && rel >= 0 && rel < kWaveV && ((rel >> 2) & 1) == lh;
+    const bool mine = tgt[j] >= 0 && rel >= 0 && rel < NBV * 32 && ((rel >> 2) & 1) == lh;
     if (__any(mine)) {
       const int want = mine ? ((rel >> 5) * 16 + ((rel & 31) >> 3) * 4 + (rel & 3)) : -1;
 #pragma unroll
-      for (int i = 0; i < kNBV; ++i)
+      for (int i = 0; i < NBV; ++i)
 #pragma unroll
         for (int e = 0; e < 16; ++e) tx[j] = (want == i * 16 + e) ? acc[i][j][e] : tx[j];
     }
-    float bm[kNBV];  // per 32-row block maximum
+    float bm[NBV];  // per 32-row block maximum
 #pragma unroll
-    for (int i = 0; i < kNBV; ++i) {
+    for (int i = 0; i < NBV; ++i) {
       float m = acc[i][j][0];
 #pragma unroll
       for (int e = 1; e < 16; e += 2) m = fmaxf(m, fmaxf(acc[i][j][e], e + 1 < 16 ? acc[i][j][e + 1] : acc[i][j][e]));
@@ -132,7 +137,7 @@ __device__ __forceinline__ void fold_tile(f32x16 (&acc)[kNBV][kNBT], RowStat (&s
     float cm = st[j].mx;
     int bi = st[j].bi;
 #pragma unroll
-    for (int i = 0; i < kNBV; ++i) {
+    for (int i = 0; i < NBV; ++i) {
       const bool up = bm[i] > cm;
       bi = up ? (vw0 + i * 32) : bi;  // first row of the 32-row block
       cm = fmaxf(cm, bm[i]);
@@ -141,7 +146,7 @@ __device__ __forceinline__ void fold_tile(f32x16 (&acc)[kNBV][kNBT], RowStat (&s
     const float m = cm * scale;
     float s0 = st[j].s * resc, s1 = 0.f, w0 = ENT ? st[j].w * resc : 0.f, w1 = 0.f;
 #pragma unroll
-    for (int i = 0; i < kNBV; ++i)
+    for (int i = 0; i < NBV; ++i)
 #pragma unroll
       for (int e = 0; e < 16; e += 2) {
         const float x0 = acc[i][j][e], x1 = acc[i][j][e + 1];
@@ -162,11 +167,12 @@ __device__ __forceinline__ void fold_tile(f32x16 (&acc)[kNBV][kNBT], RowStat (&s
 }
 
 // Merge the two lane halves that share a token and write one partial per (token, part).
-__device__ __forceinline__ void write_partials(RowStat (&st)[kNBT], float (&tx)[kNBT], FusedPartial* partials,
+template <int NBT>
+__device__ __forceinline__ void write_partials(RowStat (&st)[NBT], float (&tx)[NBT], FusedPartial* partials,
                                                int p0, int n_valid, int part, int n_parts, int l32, int lh,
                                                float scale) {
 #pragma unroll
-  for (int j = 0; j < kNBT; ++j) {
+  for (int j = 0; j < NBT; ++j) {
     stat_wave_step<5>(st[j], scale);
     const float txo = wave_exchange<5>(tx[j]);
     tx[j] = fmaxf(tx[j], txo);
@@ -420,12 +426,15 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 
   // One of the four DMA instructions of the next request (0,1: W rows; 2,3: hidden rows).
   auto issue_piece = [&](int piece) {
-    char* dst = smem + (issued & (k2Slabs - 1)) * k2SlabBytes + wave * 1024;
+    // Past the last slab the request is repeated (same addresses, same slot, identical bytes): it is
+    // issued on every step so that the code has no branch and the wait counts stay static.
+    char* dst = smem + ((issued < n_steps ? issued : n_steps - 1) & (k2Slabs - 1)) * k2SlabBytes + wave * 1024;
     if (piece < k2Loads) dma16(pa[piece], dst + piece * 8192);
     else dma16(pb[piece - k2Loads], dst + k2BV * k2RowBytes + (piece - k2Loads) * 8192);
   };
   auto issue_done = [&]() {
     ++issued;
+    if (issued >= n_steps) return;  // the stream stays on the last slab
     if (++i_kt < nk) {
 #pragma unroll
       for (int j = 0; j < k2Loads; ++j) {
@@ -455,8 +464,8 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
       fb[j] = *reinterpret_cast<const bf16x8*>(slab + rdB + j * 32 * k2RowBytes + sw);
   };
 
-  for (int q = 0; q < 3 && q < n_steps; ++q) issue();
-  wait_slabs(issued - 1);
+  for (int q = 0; q < 3; ++q) issue();
+  wait_slabs(2);
   __syncthreads();
 
   bf16x8 fa0[kNBV], fb0[kNBT], fa1[kNBV], fb1[kNBT];
@@ -473,41 +482,46 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   int step = 0;
   for (int vt = vt0; vt < vt1; ++vt) {
     for (int kt = 0; kt < nk; ++kt, ++step) {
-      // Scheduling fences pin the software pipeline; left alone, the scheduler sinks every LDS
-      // read next to its use and serialises read latency with the MFMAs.
+      // Each half-step is one scheduling region, and the group barriers ask for one LDS read (or DMA
+      // request) behind every MFMA, so that its issue hides under the 32 cycles the MFMA executes.
+      // Left alone, the scheduler sinks every LDS read next to its use; issued as a clump, the
+      // reads of all eight (barrier-aligned) waves leave the matrix pipes idle together.
       __builtin_amdgcn_sched_barrier(0);
       read_frags(step, swz1, fa1, fb1);
-      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < kNBV; ++i)
 #pragma unroll
         for (int j = 0; j < kNBT; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0[i], fb0[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int q = 0; q < kNBV + kNBT; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+      }
       __builtin_amdgcn_sched_barrier(0);
       // Slab step+1 has landed for this wave; after the (fence-less) barrier it has for everyone,
       // and everyone is past step-1, whose ring slot the next request overwrites.
-      wait_slabs(issued - (step + 2));
+      wait_slabs(1);  // steady state: slabs step+2 is the only one still allowed in flight
       __builtin_amdgcn_s_barrier();
-      const bool more = issued < n_steps;
+      // Second half: fragments of slab step+1 (after the last step a stale slot, unused) and the
+      // four DMA instructions of the next request, one per two MFMAs.
       __builtin_amdgcn_sched_barrier(0);
-      // Unconditional (after the last step it re-reads a stale slot, unused): a branch here
-      // makes the wait-count insertion treat these reads as possibly absent and drain them.
       read_frags(step + 1, swz0, fa0, fb0);
-      __builtin_amdgcn_sched_barrier(0);
-      // The next request is spread over the MFMAs (one DMA instruction per two MFMAs): all eight
-      // waves leave the barrier together, and a burst of 32 KB requests would back up the
-      // address queue and stall the in-order waves in front of their MFMAs.
 #pragma unroll
-      for (int i = 0; i < kNBV; ++i) {
+      for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
+#pragma unroll
+      for (int i = 0; i < kNBV; ++i)
 #pragma unroll
         for (int j = 0; j < kNBT; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1[i], fb1[j], acc[i][j], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        if (more) issue_piece(i);
-        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int q = 0; q < kNBV + kNBT; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+        if ((q & 1) == 0 && q < 2 * k2DmaPerSlab) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM
       }
-      if (more) issue_done();
       __builtin_amdgcn_sched_barrier(0);
+      issue_done();
     }
     const int v0 = vt * k2BV;
     fold_tile<ENT>(acc, st, tx, tgt, v0 + wave_v * kWaveV, lh, v0 + k2BV > a.V, a.V, a.scale);
@@ -520,6 +534,234 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   }
 
   write_partials(st, tx, a.partials, t0 + wave_t * kWaveT, n_valid, split * kPartsPerSplit + wave_v,
+                 sch.n_splits * kPartsPerSplit, l32, lh, a.scale);
+}
+
+// ===============================================================================================
+// Wide path (H % 128 == 0): 256 lanes = one wave per SIMD, 256 x 256 tile, 128 x 128 wave tiles.
+//
+//   * 4 waves as 2 (vocab) x 2 (token).  A wave owns 4 x 4 accumulator blocks (256 registers, which
+//     the compiler keeps in AGPRs), so each fragment read from LDS feeds four MFMAs instead of
+//     two or four of the 2-waves-per-SIMD layouts: a third fewer LDS bytes per MFMA.
+//   * K slabs are 64 wide (128-byte rows, whole cache lines per request).  With one wave per SIMD
+//     the other 256 VGPRs are free, and two of the slabs in flight live there: slab s+2 is loaded
+//     global -> registers during step s, written registers -> LDS during step s+1 and multiplied
+//     in step s+2, so a load has more than a full step (64 MFMAs per wave) to arrive.  LDS holds
+//     two 64 KB slabs, XOR-swizzled like the DMA path (chunk c of row r at c ^ ((r >> 1) & 7)).
+//   * Two fence-less barriers per step, neither followed by a dependent LDS read: B1 (after
+//     sub-step 0) says everybody is done with slab s-1, whose slot the writes of sub-steps 1-2
+//     then refill; B2 (after sub-step 2) publishes slab s+1 before sub-step 3 prefetches its first
+//     fragments.  The MFMA stream runs through step and vocab-tile boundaries without a bubble.
+// ===============================================================================================
+constexpr int k3WG = 256;
+constexpr int k3BV = 256, k3BT = 256, k3BK = 64;
+constexpr int k3WaveV = 128, k3WaveT = 128;
+constexpr int k3NBV = k3WaveV / 32, k3NBT = k3WaveT / 32;
+constexpr int k3RowBytes = k3BK * 2;                      // 128
+constexpr int k3SlabBytes = (k3BV + k3BT) * k3RowBytes;   // 65536
+constexpr int k3LdsTotal = 2 * k3SlabBytes;
+constexpr int k3Loads = k3BV * 8 / k3WG;                  // 16-byte loads per lane, operand and slab (8)
+
+template <bool ENT>
+__global__ __launch_bounds__(k3WG) void fused_lmhead_wide_kernel(FusedArgs a) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
+  const FusedSchedule sch = fused_schedule(n_valid, k3BT, a.slots, a.n_vtiles);
+  int bid = blockIdx.x;
+  if (n_valid <= 0 || bid >= sch.n_wg) return;  // the grid is sized for the worst case over n_valid
+  if ((sch.n_wg & 7) == 0) bid = (bid & 7) * (sch.n_wg >> 3) + (bid >> 3);  // contiguous logical ids per XCD
+  const int ttile = bid / sch.n_splits;
+  const int split = bid % sch.n_splits;
+  const int t0 = ttile * k3BT;
+  const int vt0 = (int)((int64_t)split * a.n_vtiles / sch.n_splits);
+  const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / sch.n_splits);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wave_v = wave & 1, wave_t = wave >> 1;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  // ---- staging assignment: load j of wave w covers tile rows (j*4 + w)*8 .. +7 of an operand ------
+  const int dr = lane >> 3;                                     // row inside the 8-row group
+  const int dc = (lane & 7) ^ (((wave & 1) << 2) | (dr >> 1));  // global chunk: position ^ ((row >> 1) & 7)
+  const __amdgpu_buffer_rsrc_t rsrcB = make_rsrc(a.hidden, a.hidden_bytes);
+  uint32_t aoff[k3Loads], boff[k3Loads];
+#pragma unroll
+  for (int j = 0; j < k3Loads; ++j) {
+    const int r = (j * 4 + wave) * 8 + dr;
+    aoff[j] = (uint32_t)r * a.weight_stride_b + dc * 16;
+    int p = t0 + r;
+    p = p < n_valid ? p : n_valid - 1;
+    const int tok = a.row_index ? a.row_index[p] : p;
+    boff[j] = (uint32_t)tok * a.hidden_stride_b + dc * 16;
+  }
+  const int st_off = wave * 1024 + lane * 16;  // where this lane's 16 bytes of load j land: + j * 4096
+
+  RowStat st[k3NBT];
+  float tx[k3NBT];
+  int tgt[k3NBT];
+#pragma unroll
+  for (int bt = 0; bt < k3NBT; ++bt) {
+    st[bt] = stat_identity();
+    tx[bt] = -INFINITY;
+    const int p = t0 + wave_t * k3WaveT + bt * 32 + l32;
+    int t = -1;
+    if (p < n_valid) t = a.targets[a.row_index ? a.row_index[p] : p];
+    tgt[bt] = (t >= 0 && t < a.V) ? t : -1;
+  }
+
+  // ---- fragment read offsets inside a slab (swizzled) --------------------------------------------
+  const int x7 = (l32 >> 1) & 7;
+  int swz[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) swz[ks] = ((ks * 2 + lh) ^ x7) * 16;
+  const int rdA = (wave_v * k3WaveV + l32) * k3RowBytes;
+  const int rdB = k3BV * k3RowBytes + (wave_t * k3WaveT + l32) * k3RowBytes;
+
+  const int nk = a.H / k3BK;
+
+  // The load stream runs two slabs ahead of the multiply; it keeps its own (tile, slab) position.
+  int l_kt = 0, l_vt = vt0;
+  __amdgpu_buffer_rsrc_t rsrcA =
+      make_rsrc(a.weight + (int64_t)l_vt * k3BV * a.weight_stride_b, (uint32_t)(a.V - l_vt * k3BV) * a.weight_stride_b);
+  // Two register sets for W (a set is written to LDS one step after it was loaded), one for hidden
+  // (its write, sub-step 2, precedes its next load, sub-step 3).  The sets are separate arrays picked
+  // at compile time: a run-time index would push them into private memory.
+  u32x4 ra0[k3Loads], ra1[k3Loads], rb[k3Loads];
+  auto load_w = [&](u32x4 (&ra)[k3Loads]) {  // W rows of slab (l_vt, l_kt)
+    const uint32_t koff = (uint32_t)l_kt * k3RowBytes;
+#pragma unroll
+    for (int j = 0; j < k3Loads; ++j) ra[j] = ld16(rsrcA, aoff[j], koff);
+  };
+  auto load_h = [&]() {  // hidden rows of the same slab
+    const uint32_t koff = (uint32_t)l_kt * k3RowBytes;
+#pragma unroll
+    for (int j = 0; j < k3Loads; ++j) rb[j] = ld16(rsrcB, boff[j], koff);
+  };
+  auto load_advance = [&]() {  // past the last slab the stream stays on it: the loads below are issued
+    if (l_vt == vt1 - 1 && l_kt == nk - 1) return;  // unconditionally, and re-reading it is harmless
+    if (++l_kt == nk) {
+      l_kt = 0;
+      ++l_vt;
+      rsrcA = make_rsrc(a.weight + (int64_t)l_vt * k3BV * a.weight_stride_b,
+                        (uint32_t)(a.V - l_vt * k3BV) * a.weight_stride_b);
+    }
+  };
+  auto write_w = [&](const u32x4 (&ra)[k3Loads], int slot) {
+    char* dst = smem + slot * k3SlabBytes + st_off;
+#pragma unroll
+    for (int j = 0; j < k3Loads; ++j) *reinterpret_cast<u32x4*>(dst + j * 4096) = ra[j];
+  };
+  auto write_h = [&](int slot) {
+    char* dst = smem + slot * k3SlabBytes + st_off + k3BV * k3RowBytes;
+#pragma unroll
+    for (int j = 0; j < k3Loads; ++j) *reinterpret_cast<u32x4*>(dst + j * 4096) = rb[j];
+  };
+  auto read_frags = [&](int slot, int ks, bf16x8 (&fa)[k3NBV], bf16x8 (&fb)[k3NBT]) {
+    const char* slab = smem + slot * k3SlabBytes;
+#pragma unroll
+    for (int i = 0; i < k3NBV; ++i)
+      fa[i] = *reinterpret_cast<const bf16x8*>(slab + rdA + i * 32 * k3RowBytes + swz[ks]);
+#pragma unroll
+    for (int j = 0; j < k3NBT; ++j)
+      fb[j] = *reinterpret_cast<const bf16x8*>(slab + rdB + j * 32 * k3RowBytes + swz[ks]);
+  };
+
+  // ---- prologue: slab 0 through registers into LDS slot 0, slab 1 into register set 1 --------------
+  load_w(ra0);
+  load_h();
+  load_advance();
+  write_w(ra0, 0);
+  write_h(0);
+  load_w(ra1);
+  load_h();
+  load_advance();
+  __syncthreads();
+
+  bf16x8 fa0[k3NBV], fb0[k3NBT], fa1[k3NBV], fb1[k3NBT];
+  read_frags(0, 0, fa0, fb0);
+
+  f32x16 acc[k3NBV][k3NBT];
+#pragma unroll
+  for (int i = 0; i < k3NBV; ++i)
+#pragma unroll
+    for (int j = 0; j < k3NBT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+#define TOME_MFMA_BLOCK(FA, FB)                                                                    \
+  _Pragma("unroll") for (int i = 0; i < k3NBV; ++i) _Pragma("unroll") for (int j = 0; j < k3NBT; ++j) \
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FA[i], FB[j], acc[i][j], 0, 0, 0)
+
+  // One K slab s.  ra_cur is the W register set that held slab s (free now, receives slab s+2),
+  // ra_nxt holds slab s+1; `cur` is the LDS slot of slab s.
+  auto do_step = [&](u32x4 (&ra_cur)[k3Loads], u32x4 (&ra_nxt)[k3Loads], int cur) {
+    const int nxt = cur ^ 1;
+    // Every load and LDS write below is issued on every step, also when the slab it belongs to does
+    // not exist any more (then it moves stale data into a slot nobody reads): under a branch the
+    // wait-count insertion must assume the newest loads may be absent and drains them all.
+    // Each sub-step is one scheduling region: 16 MFMAs, 8 fragment reads for the next sub-step and 8
+    // staging instructions.  The group barriers ask for one memory instruction behind every MFMA, so
+    // that its issue time hides under the 32 cycles the MFMA executes; issued as a clump they would
+    // leave the matrix pipe idle (one wave per SIMD: nobody else fills the gap).
+#define TOME_INTERLEAVE(MEM_MASK)                                    \
+  _Pragma("unroll") for (int q = 0; q < 8; ++q) {                    \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* MFMA */    \
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); /* DS read */ \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               \
+    __builtin_amdgcn_sched_group_barrier(MEM_MASK, 1, 0);            \
+  }
+    // sub-step 0: fragments of k1; W rows of slab step+2
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(cur, 1, fa1, fb1);
+    load_w(ra_cur);
+    TOME_MFMA_BLOCK(fa0, fb0);
+    TOME_INTERLEAVE(0x020)
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();  // B1: nobody reads slab step-1 any more; its slot may be refilled
+    // sub-step 1: fragments of k2; W half of slab step+1 goes registers -> LDS
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(cur, 2, fa0, fb0);
+    write_w(ra_nxt, nxt);
+    TOME_MFMA_BLOCK(fa1, fb1);
+    TOME_INTERLEAVE(0x200)
+    // sub-step 2: fragments of k3; hidden half of slab step+1
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(cur, 3, fa1, fb1);
+    write_h(nxt);
+    TOME_MFMA_BLOCK(fa0, fb0);
+    TOME_INTERLEAVE(0x200)
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's LDS writes are done
+    __builtin_amdgcn_s_barrier();                        // B2: slab step+1 is complete and visible
+    // sub-step 3: first fragments of slab step+1 (a stale slot after the last step, unused);
+    // hidden rows of slab step+2
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(nxt, 0, fa0, fb0);
+    load_h();
+    load_advance();
+    TOME_MFMA_BLOCK(fa1, fb1);
+    TOME_INTERLEAVE(0x020)
+    __builtin_amdgcn_sched_barrier(0);
+#undef TOME_INTERLEAVE
+  };
+  for (int vt = vt0; vt < vt1; ++vt) {
+    for (int kt = 0; kt < nk; kt += 2) {  // nk is even (H % 128 == 0): slab parity == kt parity
+      do_step(ra0, ra1, 0);
+      do_step(ra1, ra0, 1);
+    }
+    const int v0 = vt * k3BV;
+    fold_tile<ENT>(acc, st, tx, tgt, v0 + wave_v * k3WaveV, lh, v0 + k3BV > a.V, a.V, a.scale);
+#pragma unroll
+    for (int i = 0; i < k3NBV; ++i)
+#pragma unroll
+      for (int j = 0; j < k3NBT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  }
+#undef TOME_MFMA_BLOCK
+
+  write_partials(st, tx, a.partials, t0 + wave_t * k3WaveT, n_valid, split * kPartsPerSplit + wave_v,
                  sch.n_splits * kPartsPerSplit, l32, lh, a.scale);
 }
 
@@ -685,12 +927,13 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
 }
 
 // ---- host side -----------------------------------------------------------------------------------
-// The DMA kernel needs whole 32-wide K slabs and pays for 256-token tiles; short batches and
-// ragged H go to the generic kernel.
-static bool use_dma_kernel(int64_t n_tokens, int64_t H) { return H % k2BK == 0 && n_tokens > kBT; }
+// The wide and DMA kernels need whole 64- / 32-wide K slabs and pay for 256-token tiles; short
+// batches and ragged H go to the generic kernel.
+
+enum FusedKind { kGeneric = 0, kDma = 1, kWide = 2 };
 
 struct FusedPlan {
-  bool dma;
+  FusedKind kind;
   int bt, bv, slots, n_vtiles;
   int grid;            // workgroups to launch: the most any number of valid tokens can ask for
   size_t max_records;  // partial records any number of valid tokens can produce
@@ -698,10 +941,19 @@ struct FusedPlan {
 
 static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   FusedPlan p;
-  p.dma = use_dma_kernel(n_tokens, H);
-  p.bt = p.dma ? k2BT : kBT;
-  p.bv = p.dma ? k2BV : kBV;
-  p.slots = p.dma ? 256 : 512;  // resident workgroups on 256 CUs: 1 per CU (128 KB LDS) or 2
+  p.kind = kGeneric;
+  // Measured on MI355X: the wide path wins from H = 4096 up (its exposed epilogue costs more than its
+  // leaner K loop gains on short K), the DMA path below.
+  if (n_tokens > kBT && H >= 4096 && H % (2 * k3BK) == 0) p.kind = kWide;
+  else if (n_tokens > kBT && H % k2BK == 0) p.kind = kDma;
+  if (const char* ov = getenv("TOME_FUSED_KERNEL")) {  // tuning knob: force a path where its shape rules allow
+    if (ov[0] == 'g') p.kind = kGeneric;
+    if (ov[0] == 'd' && H % k2BK == 0) p.kind = kDma;
+    if (ov[0] == 'w' && H % (2 * k3BK) == 0) p.kind = kWide;
+  }
+  p.bt = p.kind == kGeneric ? kBT : k2BT;   // the DMA and wide paths share the 256 x 256 tile
+  p.bv = p.kind == kGeneric ? kBV : k2BV;
+  p.slots = p.kind == kGeneric ? 512 : 256;  // resident workgroups on 256 CUs: 2 per CU, or 1 (128 KB LDS)
   p.n_vtiles = (int)((V + p.bv - 1) / p.bv);
   p.grid = 0;
   p.max_records = 0;
@@ -726,20 +978,25 @@ size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weigh
   return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, H, V);
 }
 
+template <typename K>
+static void allow_big_lds(K kernel, int bytes) {
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
 template <bool ENT>
-static void launch_main(const FusedArgs& a, bool dma, int grid, hipStream_t stream) {
-  if (dma) {
-    static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
-    if (!attr_set) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fused_lmhead_dma_kernel<ENT>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, k2LdsTotal);
-      attr_set = true;
-    }
-    hipLaunchKernelGGL(fused_lmhead_dma_kernel<ENT>, dim3((unsigned)grid), dim3(k2WG),
-                       k2LdsTotal, stream, a);
+static void launch_main(const FusedArgs& a, FusedKind kind, int grid, hipStream_t stream) {
+  static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
+  if (!attr_set) {
+    allow_big_lds(&fused_lmhead_dma_kernel<ENT>, k2LdsTotal);
+    allow_big_lds(&fused_lmhead_wide_kernel<ENT>, k3LdsTotal);
+    attr_set = true;
+  }
+  if (kind == kWide) {
+    hipLaunchKernelGGL(fused_lmhead_wide_kernel<ENT>, dim3((unsigned)grid), dim3(k3WG), k3LdsTotal, stream, a);
+  } else if (kind == kDma) {
+    hipLaunchKernelGGL(fused_lmhead_dma_kernel<ENT>, dim3((unsigned)grid), dim3(k2WG), k2LdsTotal, stream, a);
   } else {
-    hipLaunchKernelGGL(fused_lmhead_kernel<ENT>, dim3((unsigned)grid), dim3(kFusedWG), 0,
-                       stream, a);
+    hipLaunchKernelGGL(fused_lmhead_kernel<ENT>, dim3((unsigned)grid), dim3(kFusedWG), 0, stream, a);
   }
 }
 
@@ -775,7 +1032,6 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w
   a.H = (int)H;
   a.V = (int)V;
   const FusedPlan plan = fused_plan(n_tokens, H, V);
-  const bool dma = plan.dma;
   a.n_vtiles = plan.n_vtiles;
   a.slots = plan.slots;
   a.scale = kLog2e / temperature;
@@ -784,12 +1040,12 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w
 
   a.weight = static_cast<const char*>(w0);
   a.partials = p0;
-  if (out_entropy) launch_main<true>(a, dma, plan.grid, stream);
-  else launch_main<false>(a, dma, plan.grid, stream);
+  if (out_entropy) launch_main<true>(a, plan.kind, plan.grid, stream);
+  else launch_main<false>(a, plan.kind, plan.grid, stream);
   if (w1) {
     a.weight = static_cast<const char*>(w1);
     a.partials = p1;
-    launch_main<false>(a, dma, plan.grid, stream);
+    launch_main<false>(a, plan.kind, plan.grid, stream);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
