@@ -310,21 +310,117 @@ __global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) 
 }
 
 
+
+// ---- 16x16x32 MFMA accumulator layout --------------------------------------------------------------
+// A 16x16 block lives in four registers: lane l holds token column l % 16 and vocab rows
+// 4*(l/16) + e, e = 0..3.  A lane therefore owns one token per 16-token block, and the four lane
+// groups l/16 share that token: they are merged once, at the end, over lane ^ 16 and lane ^ 32.
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+// Fold one wave tile (NBV x NBT blocks of 16x16) into the per-token running states.  Element e of
+// block i holds vocab row  vw0 + i*16 + 4*g + e  (g = lane / 16) for the token of block column j.
+template <bool ENT, int NBV, int NBT>
+__device__ __forceinline__ void fold_tile16(f32x4v (&acc)[NBV][NBT], RowStat (&st)[NBT], float (&tx)[NBT],
+                                            const int (&tgt)[NBT], int vw0, int g, bool partial_tile, int V,
+                                            float scale) {
+  if (partial_tile) {  // last vocab tile: rows past V do not exist
+#pragma unroll
+    for (int i = 0; i < NBV; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool dead = vw0 + i * 16 + 4 * g + e >= V;
+#pragma unroll
+        for (int j = 0; j < NBT; ++j) acc[i][j][e] = dead ? -INFINITY : acc[i][j][e];
+      }
+  }
+#pragma unroll
+  for (int j = 0; j < NBT; ++j) {
+    __builtin_amdgcn_sched_barrier(0);  // one scheduling region per token block (register pressure)
+    // Target capture: rare (one tile in V/256 per token), so behind a wave-uniform test.
+    const int rel = tgt[j] - vw0;
+    const bool mine = tgt[j] >= 0 && rel >= 0 && rel < NBV * 16 && ((rel >> 2) & 3) == g;
+    if (__any(mine)) {
+      const int want = mine ? ((rel >> 4) * 4 + (rel & 3)) : -1;
+#pragma unroll
+      for (int i = 0; i < NBV; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) tx[j] = (want == i * 4 + e) ? acc[i][j][e] : tx[j];
+    }
+    float cm = st[j].mx;
+    int bi = st[j].bi;
+#pragma unroll
+    for (int i = 0; i < NBV; ++i) {
+      const float bm = fmaxf(fmaxf(acc[i][j][0], acc[i][j][1]), fmaxf(acc[i][j][2], acc[i][j][3]));
+      const bool up = bm > cm;
+      bi = up ? (vw0 + i * 16) : bi;  // first row of the 16-row block
+      cm = fmaxf(cm, bm);
+    }
+    const float resc = fast_exp2((st[j].mx - cm) * scale);
+    const float m = cm * scale;
+    float s0 = st[j].s * resc, s1 = 0.f, w0 = ENT ? st[j].w * resc : 0.f, w1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NBV; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; e += 2) {
+        const float x0 = acc[i][j][e], x1 = acc[i][j][e + 1];
+        const float e0 = fast_exp2(fmaf(x0, scale, -m));
+        const float e1 = fast_exp2(fmaf(x1, scale, -m));
+        s0 += e0;
+        s1 += e1;
+        if constexpr (ENT) {
+          w0 = fmaf(fmaxf(x0, kMaxFloor) * scale, e0, w0);
+          w1 = fmaf(fmaxf(x1, kMaxFloor) * scale, e1, w1);
+        }
+      }
+    st[j].mx = cm;
+    st[j].bi = bi;
+    st[j].s = s0 + s1;
+    if constexpr (ENT) st[j].w = w0 + w1;
+  }
+}
+
+// Merge the four lane groups that share a token and write one partial per (token, part).
+template <int NBT>
+__device__ __forceinline__ void write_partials16(RowStat (&st)[NBT], float (&tx)[NBT], FusedPartial* partials,
+                                                 int p0, int n_valid, int part, int n_parts, int l16, int g,
+                                                 float scale) {
+#pragma unroll
+  for (int j = 0; j < NBT; ++j) {
+    stat_wave_step<4>(st[j], scale);
+    stat_wave_step<5>(st[j], scale);
+    tx[j] = fmaxf(tx[j], wave_exchange<4>(tx[j]));
+    tx[j] = fmaxf(tx[j], wave_exchange<5>(tx[j]));
+    const int p = p0 + j * 16 + l16;
+    if (g == 0 && p < n_valid) {
+      FusedPartial out;
+      out.mx = st[j].mx;
+      out.s = st[j].s;
+      out.w = st[j].w;
+      out.tx = tx[j];
+      out.bi = st[j].bi;
+      out.pad[0] = out.pad[1] = out.pad[2] = 0;
+      partials[(int64_t)p * n_parts + part] = out;
+    }
+  }
+}
+
 // ===============================================================================================
-// Fast path (H % 32 == 0): 512 lanes, 256 x 256 tile, K slabs DMA'd straight into LDS through a
-// four-slab ring.
+// Fast path (H % 64 == 0): 512 lanes, 256 x 256 tile, v_mfma_f32_16x16x32_bf16, K slabs DMA'd straight
+// into LDS through a four-slab ring.
 //
-//   * 8 waves as 2 (vocab) x 4 (token); the per-wave tile is still 128 vocab x 64 tokens, so
-//     fold_tile / write_partials and the partial layout are shared with the generic kernel.
+//   * 8 waves as 2 (vocab) x 4 (token), 128 vocab x 64 tokens per wave as 8 x 4 blocks of 16x16.  The
+//     16x16x32 MFMA moves half the accumulator bytes per FLOP of the 32x32x16 one; on this
+//     power-limited part that alone is worth 12-16 % (measured with the instruction swapped in place).
+//     The partial layout is shared with the other kernels.
 //   * global_load_lds_dwordx4: every lane fetches 16 bytes and the wave's 1 KB lands contiguously
 //     in LDS, bypassing registers.  No staging registers are needed, which leaves room to
 //     double-buffer the MFMA fragments.
 //   * What bounds this kernel is the L2 -> LDS fill (64 KB per 256x256x64 MACs and CU): measured
 //     alone, with one slab in flight, it takes as long as the MFMAs.  Hence a ring of four 32 KB
 //     slabs (K = 32 each: W 256 rows + hidden 256 rows, 64 bytes per row) with three requests in
-//     flight.  Step s (one slab = two MFMA sub-steps) runs
-//         reads(s, k1) | MFMA(s, k0) | wait slab s+1, barrier, request slab s+3 |
-//         reads(s+1, k0) | MFMA(s, k1)
+//     flight.  Step s (one slab = one K = 32 MFMA step, 32 MFMAs per wave in two halves) runs
+//         reads(s, W blocks 4-7) | MFMA(s, blocks 0-3) | wait slab s+1, barrier, request slab s+3 |
+//         reads(s+1, W blocks 0-3 and hidden) | MFMA(s, blocks 4-7)
 //     The barrier sits mid-step: everybody is then past step s-1, so its slab can be refilled,
 //     and slab s+1 is visible before its first fragments are read, which happens under the
 //     second half of the MFMAs - the MFMA stream has no bubble at step or vocab-tile boundaries.
@@ -342,6 +438,7 @@ constexpr int k2Slabs = 4;
 constexpr int k2LdsTotal = k2Slabs * k2SlabBytes;        // 131072
 constexpr int k2Loads = k2BV * (k2RowBytes / 16) / k2WG; // DMA instructions per lane, operand and slab (2)
 constexpr int k2DmaPerSlab = 2 * k2Loads;                // vmcnt units per slab and wave
+constexpr int k2NBV = kWaveV / 16, k2NBT = kWaveT / 16;  // 16x16 blocks per wave tile: 8 x 4
 
 __device__ __forceinline__ void dma16(const char* gptr, char* lds_wave_base) {
   __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(gptr),
@@ -354,7 +451,7 @@ __device__ __forceinline__ void wait_slabs(int slabs) {
   else if (slabs == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
-static_assert(k2DmaPerSlab == 4 && kNBV == 4, "wait_slabs and the DMA interleave assume 4 DMA instructions per slab");
+static_assert(k2DmaPerSlab == 4 && k2NBV == 8 && k2NBT == 4, "wait_slabs and the MFMA/DMA interleave are written for this shape");
 
 template <bool ENT>
 __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
@@ -371,9 +468,10 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   const int vt0 = (int)((int64_t)split * a.n_vtiles / sch.n_splits);
   const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / sch.n_splits);
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps LDS bases scalar
   const int wave_v = wave & 1, wave_t = wave >> 1;
-  const int l32 = lane & 31, lh = lane >> 5;
+  const int l16 = lane & 15, g = lane >> 4;  // 16x16 MFMA: token column, lane group
 
   // ---- DMA assignment: instruction j of wave w fills LDS rows (j*8 + w)*16 .. +15 of an operand --
   // All address arithmetic is incremental: per-lane pointers advance by one slab (64 bytes) per
@@ -399,24 +497,24 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     pb[j] = a.hidden + (int64_t)tok * a.hidden_stride_b + dc * 16;
   }
 
-  RowStat st[kNBT];
-  float tx[kNBT];
-  int tgt[kNBT];
+  // ---- per-lane token state: one token per 16-token block, shared by the four lane groups ---------
+  RowStat st[k2NBT];
+  float tx[k2NBT];
+  int tgt[k2NBT];
 #pragma unroll
-  for (int bt = 0; bt < kNBT; ++bt) {
+  for (int bt = 0; bt < k2NBT; ++bt) {
     st[bt] = stat_identity();
     tx[bt] = -INFINITY;
-    const int p = t0 + wave_t * kWaveT + bt * 32 + l32;
+    const int p = t0 + wave_t * kWaveT + bt * 16 + l16;
     int t = -1;
     if (p < n_valid) t = a.targets[a.row_index ? a.row_index[p] : p];
     tgt[bt] = (t >= 0 && t < a.V) ? t : -1;
   }
 
-  // ---- fragment read offsets inside a slab (swizzled) --------------------------------------------
-  const int x3 = (l32 >> 2) & 3;
-  const int swz0 = ((0 + lh) ^ x3) * 16, swz1 = ((2 + lh) ^ x3) * 16;
-  const int rdA = (wave_v * kWaveV + l32) * k2RowBytes;
-  const int rdB = k2BV * k2RowBytes + (wave_t * kWaveT + l32) * k2RowBytes;
+  // ---- fragment read offsets inside a slab (swizzled): lane group g reads 16-byte chunk g --------
+  const int swz = (g ^ ((l16 >> 2) & 3)) * 16;
+  const int rdA = (wave_v * kWaveV + l16) * k2RowBytes + swz;
+  const int rdB = k2BV * k2RowBytes + (wave_t * kWaveT + l16) * k2RowBytes + swz;
 
   const int nk = a.H / k2BK;
   const int n_steps = (vt1 - vt0) * nk;
@@ -454,87 +552,101 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
     issue_done();
   };
-  auto read_frags = [&](int step, int sw, bf16x8 (&fa)[kNBV], bf16x8 (&fb)[kNBT]) {
-    const char* slab = smem + (step & (k2Slabs - 1)) * k2SlabBytes;
+  // Fragments of one slab: W blocks [i0, i0 + 4) and / or the four hidden blocks.
+  auto read_a = [&](int slot, int i0, bf16x8 (&fa)[4]) {
+    const char* slab = smem + (slot & (k2Slabs - 1)) * k2SlabBytes;
 #pragma unroll
-    for (int i = 0; i < kNBV; ++i)
-      fa[i] = *reinterpret_cast<const bf16x8*>(slab + rdA + i * 32 * k2RowBytes + sw);
+    for (int i = 0; i < 4; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(slab + rdA + (i0 + i) * 16 * k2RowBytes);
+  };
+  auto read_b = [&](int slot, bf16x8 (&fb)[k2NBT]) {
+    const char* slab = smem + (slot & (k2Slabs - 1)) * k2SlabBytes;
 #pragma unroll
-    for (int j = 0; j < kNBT; ++j)
-      fb[j] = *reinterpret_cast<const bf16x8*>(slab + rdB + j * 32 * k2RowBytes + sw);
+    for (int j = 0; j < k2NBT; ++j) fb[j] = *reinterpret_cast<const bf16x8*>(slab + rdB + j * 16 * k2RowBytes);
   };
 
   for (int q = 0; q < 3; ++q) issue();
   wait_slabs(2);
   __syncthreads();
 
-  bf16x8 fa0[kNBV], fb0[kNBT], fa1[kNBV], fb1[kNBT];
-  read_frags(0, swz0, fa0, fb0);
+  bf16x8 fa_lo[4], fa_hi[4], fb0[k2NBT], fb1[k2NBT];
+  read_a(0, 0, fa_lo);
+  read_b(0, fb0);
 
-  f32x16 acc[kNBV][kNBT];
+  f32x4v acc[k2NBV][k2NBT];
 #pragma unroll
-  for (int i = 0; i < kNBV; ++i)
+  for (int i = 0; i < k2NBV; ++i)
 #pragma unroll
-    for (int j = 0; j < kNBT; ++j)
+    for (int j = 0; j < k2NBT; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
   int step = 0;
+  // One slab (K = 32) = 32 MFMAs per wave in two halves of 16 (vocab blocks 0-3, then 4-7).  Each half
+  // is one scheduling region in which the group barriers put one LDS read (or DMA request) behind
+  // every MFMA, so that its issue hides under the MFMA's execution.
+  auto do_step = [&](bf16x8 (&fb_cur)[k2NBT], bf16x8 (&fb_nxt)[k2NBT]) {
+    __builtin_amdgcn_sched_barrier(0);
+    read_a(step, 4, fa_hi);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < k2NBT; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa_lo[i], fb_cur[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // Slab step+1 has landed for this wave; after the (fence-less) barrier it has for everyone, and
+    // everyone is past step-1, whose ring slot the next request overwrites.
+    wait_slabs(1);
+    __builtin_amdgcn_s_barrier();
+    // Second half: first fragments of slab step+1 (after the last step a stale slot, unused) and the
+    // four DMA instructions of the next request.
+    __builtin_amdgcn_sched_barrier(0);
+    read_a(step + 1, 0, fa_lo);
+    read_b(step + 1, fb_nxt);
+#pragma unroll
+    for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < k2NBT; ++j)
+        acc[4 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa_hi[i], fb_cur[j], acc[4 + i][j], 0, 0, 0);
+    // The DMA requests write LDS, so they keep their program order after the fragment reads.
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM (DMA request)
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    issue_done();
+    ++step;
+  };
+
   for (int vt = vt0; vt < vt1; ++vt) {
-    for (int kt = 0; kt < nk; ++kt, ++step) {
-      // Each half-step is one scheduling region, and the group barriers ask for one LDS read (or DMA
-      // request) behind every MFMA, so that its issue hides under the 32 cycles the MFMA executes.
-      // Left alone, the scheduler sinks every LDS read next to its use; issued as a clump, the
-      // reads of all eight (barrier-aligned) waves leave the matrix pipes idle together.
-      __builtin_amdgcn_sched_barrier(0);
-      read_frags(step, swz1, fa1, fb1);
-#pragma unroll
-      for (int i = 0; i < kNBV; ++i)
-#pragma unroll
-        for (int j = 0; j < kNBT; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0[i], fb0[j], acc[i][j], 0, 0, 0);
-#pragma unroll
-      for (int q = 0; q < kNBV + kNBT; ++q) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      // Slab step+1 has landed for this wave; after the (fence-less) barrier it has for everyone,
-      // and everyone is past step-1, whose ring slot the next request overwrites.
-      wait_slabs(1);  // steady state: slabs step+2 is the only one still allowed in flight
-      __builtin_amdgcn_s_barrier();
-      // Second half: fragments of slab step+1 (after the last step a stale slot, unused) and the
-      // four DMA instructions of the next request, one per two MFMAs.
-      __builtin_amdgcn_sched_barrier(0);
-      read_frags(step + 1, swz0, fa0, fb0);
-#pragma unroll
-      for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
-#pragma unroll
-      for (int i = 0; i < kNBV; ++i)
-#pragma unroll
-        for (int j = 0; j < kNBT; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1[i], fb1[j], acc[i][j], 0, 0, 0);
-#pragma unroll
-      for (int q = 0; q < kNBV + kNBT; ++q) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-        if ((q & 1) == 0 && q < 2 * k2DmaPerSlab) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      issue_done();
+    for (int kt = 0; kt < nk; kt += 2) {  // nk is even (H % 64 == 0): the hidden fragment sets alternate
+      do_step(fb0, fb1);
+      do_step(fb1, fb0);
     }
     const int v0 = vt * k2BV;
-    fold_tile<ENT>(acc, st, tx, tgt, v0 + wave_v * kWaveV, lh, v0 + k2BV > a.V, a.V, a.scale);
+    fold_tile16<ENT>(acc, st, tx, tgt, v0 + wave_v * kWaveV, g, v0 + k2BV > a.V, a.V, a.scale);
 #pragma unroll
-    for (int i = 0; i < kNBV; ++i)
+    for (int i = 0; i < k2NBV; ++i)
 #pragma unroll
-      for (int j = 0; j < kNBT; ++j)
+      for (int j = 0; j < k2NBT; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
   }
 
-  write_partials(st, tx, a.partials, t0 + wave_t * kWaveT, n_valid, split * kPartsPerSplit + wave_v,
-                 sch.n_splits * kPartsPerSplit, l32, lh, a.scale);
+  write_partials16(st, tx, a.partials, t0 + wave_t * kWaveT, n_valid, split * kPartsPerSplit + wave_v,
+                   sch.n_splits * kPartsPerSplit, l16, g, a.scale);
 }
 
 // ===============================================================================================
@@ -945,10 +1057,10 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   // Measured on MI355X: the wide path wins from H = 4096 up (its exposed epilogue costs more than its
   // leaner K loop gains on short K), the DMA path below.
   if (n_tokens > kBT && H >= 4096 && H % (2 * k3BK) == 0) p.kind = kWide;
-  else if (n_tokens > kBT && H % k2BK == 0) p.kind = kDma;
+  else if (n_tokens > kBT && H % (2 * k2BK) == 0) p.kind = kDma;
   if (const char* ov = getenv("TOME_FUSED_KERNEL")) {  // tuning knob: force a path where its shape rules allow
     if (ov[0] == 'g') p.kind = kGeneric;
-    if (ov[0] == 'd' && H % k2BK == 0) p.kind = kDma;
+    if (ov[0] == 'd' && H % (2 * k2BK) == 0) p.kind = kDma;
     if (ov[0] == 'w' && H % (2 * k3BK) == 0) p.kind = kWide;
   }
   p.bt = p.kind == kGeneric ? kBT : k2BT;   // the DMA and wide paths share the 256 x 256 tile
