@@ -406,7 +406,7 @@ __device__ __forceinline__ void write_partials16(RowStat (&st)[NBT], float (&tx)
 
 // ===============================================================================================
 // Fast path (H % 64 == 0): 512 lanes, 256 x 256 tile, v_mfma_f32_16x16x32_bf16, K slabs DMA'd straight
-// into LDS through a four-slab ring.
+// into LDS, double-buffered.
 //
 //   * 8 waves as 2 (vocab) x 4 (token), 128 vocab x 64 tokens per wave as 8 x 4 blocks of 16x16.  The
 //     16x16x32 MFMA moves half the accumulator bytes per FLOP of the 32x32x16 one; on this
@@ -415,43 +415,50 @@ __device__ __forceinline__ void write_partials16(RowStat (&st)[NBT], float (&tx)
 //   * global_load_lds_dwordx4: every lane fetches 16 bytes and the wave's 1 KB lands contiguously
 //     in LDS, bypassing registers.  No staging registers are needed, which leaves room to
 //     double-buffer the MFMA fragments.
-//   * What bounds this kernel is the L2 -> LDS fill (64 KB per 256x256x64 MACs and CU): measured
-//     alone, with one slab in flight, it takes as long as the MFMAs.  Hence a ring of four 32 KB
-//     slabs (K = 32 each: W 256 rows + hidden 256 rows, 64 bytes per row) with three requests in
-//     flight.  Step s (one slab = one K = 32 MFMA step, 32 MFMAs per wave in two halves) runs
-//         reads(s, W blocks 4-7) | MFMA(s, blocks 0-3) | wait slab s+1, barrier, request slab s+3 |
-//         reads(s+1, W blocks 0-3 and hidden) | MFMA(s, blocks 4-7)
-//     The barrier sits mid-step: everybody is then past step s-1, so its slab can be refilled,
-//     and slab s+1 is visible before its first fragments are read, which happens under the
-//     second half of the MFMAs - the MFMA stream has no bubble at step or vocab-tile boundaries.
+//   * What bounds this kernel is the L2 -> LDS fill (64 KB per 256x256x64 MACs and CU), and the L2
+//     serves it by the request, not by the byte: a slab row is therefore one whole 128-byte cache line
+//     (K = 64), which streams 1.5x faster than 64-byte rows.  Two 64 KB slabs (W 256 rows + hidden
+//     256 rows each) fill the LDS; one is computed on while the other is in flight.  Step s (one
+//     slab = two K = 32 MFMA sub-steps of 32 MFMAs per wave, each in two halves by vocab block) runs
+//         MFMA(s, k0, blocks 0-3) | reads (s, k0, blocks 4-7)
+//         MFMA(s, k0, blocks 4-7) | reads (s, k1, blocks 0-3 and hidden)
+//         MFMA(s, k1, blocks 0-3) | reads (s, k1, blocks 4-7)
+//         own reads and own share of slab s+1 complete; barrier
+//         MFMA(s, k1, blocks 4-7) | reads (s+1, k0, blocks 0-3 and hidden), request slab s+2
+//     After the barrier everybody has read all of slab s, so it can be refilled, and slab s+1 is
+//     visible before its first fragments are read, which happens under the last quarter of the
+//     MFMAs - the MFMA stream has no bubble at step or vocab-tile boundaries.
 //   * Bank conflicts are avoided by an XOR swizzle instead of padding (DMA writes are dense).
 //     The LDS has 64 four-byte banks, so a 16-lane phase of a 128-bit read is conflict-free when
-//     its 16 rows hit 16 different 16-byte bank groups.  A 64-byte row r covers groups
-//     4*(r&3) .. +3, so chunk c of row r is stored at chunk position c ^ ((r >> 2) & 3); the
-//     lane that DMA-writes position p of row r fetches global chunk p ^ ((r >> 2) & 3).
+//     its 16 rows hit 16 different 16-byte bank groups.  A 128-byte row r covers groups
+//     8*(r&1) .. +7, so chunk c of row r is stored at chunk position c ^ ((r >> 1) & 7); the
+//     lane that DMA-writes position p of row r fetches global chunk p ^ ((r >> 1) & 7).
 // ===============================================================================================
 constexpr int k2BV = 256, k2BT = 256, k2WG = 512;
-constexpr int k2BK = 32;
-constexpr int k2RowBytes = k2BK * 2;                     // 64
-constexpr int k2SlabBytes = (k2BV + k2BT) * k2RowBytes;  // 32768
-constexpr int k2Slabs = 4;
+constexpr int k2BK = 64;
+constexpr int k2RowBytes = k2BK * 2;                     // 128: one cache line
+constexpr int k2SlabBytes = (k2BV + k2BT) * k2RowBytes;  // 65536
+constexpr int k2Slabs = 2;
 constexpr int k2LdsTotal = k2Slabs * k2SlabBytes;        // 131072
-constexpr int k2Loads = k2BV * (k2RowBytes / 16) / k2WG; // DMA instructions per lane, operand and slab (2)
-constexpr int k2DmaPerSlab = 2 * k2Loads;                // vmcnt units per slab and wave
+constexpr int k2Loads = k2BV * (k2RowBytes / 16) / k2WG; // DMA instructions per lane, operand and slab (4)
+constexpr int k2DmaPerSlab = 2 * k2Loads;                // DMA instructions per slab and wave (8)
 constexpr int k2NBV = kWaveV / 16, k2NBT = kWaveT / 16;  // 16x16 blocks per wave tile: 8 x 4
+static_assert(k2DmaPerSlab == 8 && k2NBV == 8 && k2NBT == 4, "the MFMA/DMA interleave is written for this shape");
 
 __device__ __forceinline__ void dma16(const char* gptr, char* lds_wave_base) {
   __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(gptr),
                                    (__attribute__((address_space(3))) uint32_t*)lds_wave_base, 16, 0, 0);
 }
 
-// Wait until at most `slabs` of this wave's slab requests are still in flight.
-__device__ __forceinline__ void wait_slabs(int slabs) {
-  if (slabs >= 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-  else if (slabs == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+// Scheduling pattern: N_READS times (N_MFMA MFMAs, then one LDS read).
+template <int N_MFMA, int N_READS>
+__device__ __forceinline__ void pair_reads() {
+#pragma unroll
+  for (int q = 0; q < N_READS; ++q) {
+    __builtin_amdgcn_sched_group_barrier(0x008, N_MFMA, 0);  // MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);       // DS read
+  }
 }
-static_assert(k2DmaPerSlab == 4 && k2NBV == 8 && k2NBT == 4, "wait_slabs and the MFMA/DMA interleave are written for this shape");
 
 template <bool ENT>
 __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
@@ -473,17 +480,17 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   const int wave_v = wave & 1, wave_t = wave >> 1;
   const int l16 = lane & 15, g = lane >> 4;  // 16x16 MFMA: token column, lane group
 
-  // ---- DMA assignment: instruction j of wave w fills LDS rows (j*8 + w)*16 .. +15 of an operand --
-  // All address arithmetic is incremental: per-lane pointers advance by one slab (64 bytes) per
+  // ---- DMA assignment: instruction j of wave w fills LDS rows (j*8 + w)*8 .. +7 of an operand ----
+  // All address arithmetic is incremental: per-lane pointers advance by one slab (128 bytes) per
   // request and are rebased at vocab-tile changes, so a step carries no multiplies or divides.
-  const int dr = lane >> 2;                       // row inside the 16-row group
-  const int dc = (lane & 3) ^ ((dr >> 2) & 3);    // global chunk: position ^ ((row >> 2) & 3)
+  const int dr = lane >> 3;                                   // row inside the 8-row group
+  const int dc = (lane & 7) ^ (4 * (wave & 1) + (dr >> 1));   // global chunk: position ^ ((row >> 1) & 7)
   const char* pa[k2Loads];  // next W slab to request, per DMA instruction
   const char* pb[k2Loads];  // next hidden slab
   auto point_a = [&](int vt) {  // rows past V (last tile only) read the last row; masked in the epilogue
 #pragma unroll
     for (int j = 0; j < k2Loads; ++j) {
-      int64_t v = (int64_t)vt * k2BV + (j * 8 + wave) * 16 + dr;
+      int64_t v = (int64_t)vt * k2BV + (j * 8 + wave) * 8 + dr;
       v = v < a.V ? v : a.V - 1;
       pa[j] = a.weight + v * a.weight_stride_b + dc * 16;
     }
@@ -491,7 +498,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   point_a(vt0);
 #pragma unroll
   for (int j = 0; j < k2Loads; ++j) {
-    int p = t0 + (j * 8 + wave) * 16 + dr;
+    int p = t0 + (j * 8 + wave) * 8 + dr;
     p = p < n_valid ? p : n_valid - 1;
     const int tok = a.row_index ? a.row_index[p] : p;
     pb[j] = a.hidden + (int64_t)tok * a.hidden_stride_b + dc * 16;
@@ -511,8 +518,8 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     tgt[bt] = (t >= 0 && t < a.V) ? t : -1;
   }
 
-  // ---- fragment read offsets inside a slab (swizzled): lane group g reads 16-byte chunk g --------
-  const int swz = (g ^ ((l16 >> 2) & 3)) * 16;
+  // ---- fragment read offsets inside a slab (swizzled): lane group g reads chunk 4*ks + g ----------
+  const int swz = (g ^ ((l16 >> 1) & 7)) * 16;  // sub-step k0; k1 is this ^ 64
   const int rdA = (wave_v * kWaveV + l16) * k2RowBytes + swz;
   const int rdB = k2BV * k2RowBytes + (wave_t * kWaveT + l16) * k2RowBytes + swz;
 
@@ -520,11 +527,11 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   const int n_steps = (vt1 - vt0) * nk;
   const int64_t slab_rewind = (int64_t)(nk - 1) * k2RowBytes;
   int i_kt = 0, i_vt = vt0;  // slab the next `issue` will request
-  int issued = 0;            // slabs requested so far; request q lands in ring slot q % 4
+  int issued = 0;            // slabs requested so far; request q lands in buffer q % 2
 
-  // One of the four DMA instructions of the next request (0,1: W rows; 2,3: hidden rows).
+  // One of the eight DMA instructions of the next request (0-3: W rows; 4-7: hidden rows).
   auto issue_piece = [&](int piece) {
-    // Past the last slab the request is repeated (same addresses, same slot, identical bytes): it is
+    // Past the last slab the request is repeated (same addresses, same buffer, identical bytes): it is
     // issued on every step so that the code has no branch and the wait counts stay static.
     char* dst = smem + ((issued < n_steps ? issued : n_steps - 1) & (k2Slabs - 1)) * k2SlabBytes + wave * 1024;
     if (piece < k2Loads) dma16(pa[piece], dst + piece * 8192);
@@ -547,30 +554,31 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
       if (i_vt < vt1) point_a(i_vt);
     }
   };
-  auto issue = [&]() {
+  // Fragments of one K = 32 sub-step of a slab: W blocks [i0, i0 + 4) or the four hidden blocks.
+  auto read_a = [&](int slot, int ks, int i0, bf16x8 (&fa)[4]) {
+    const char* slab = smem + (slot & (k2Slabs - 1)) * k2SlabBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      fa[i] = *reinterpret_cast<const bf16x8*>(slab + (rdA ^ (ks * 64)) + (i0 + i) * 16 * k2RowBytes);
+  };
+  auto read_b = [&](int slot, int ks, bf16x8 (&fb)[k2NBT]) {
+    const char* slab = smem + (slot & (k2Slabs - 1)) * k2SlabBytes;
+#pragma unroll
+    for (int j = 0; j < k2NBT; ++j)
+      fb[j] = *reinterpret_cast<const bf16x8*>(slab + (rdB ^ (ks * 64)) + j * 16 * k2RowBytes);
+  };
+
+  for (int q = 0; q < 2; ++q) {
 #pragma unroll
     for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
     issue_done();
-  };
-  // Fragments of one slab: W blocks [i0, i0 + 4) and / or the four hidden blocks.
-  auto read_a = [&](int slot, int i0, bf16x8 (&fa)[4]) {
-    const char* slab = smem + (slot & (k2Slabs - 1)) * k2SlabBytes;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(slab + rdA + (i0 + i) * 16 * k2RowBytes);
-  };
-  auto read_b = [&](int slot, bf16x8 (&fb)[k2NBT]) {
-    const char* slab = smem + (slot & (k2Slabs - 1)) * k2SlabBytes;
-#pragma unroll
-    for (int j = 0; j < k2NBT; ++j) fb[j] = *reinterpret_cast<const bf16x8*>(slab + rdB + j * 16 * k2RowBytes);
-  };
-
-  for (int q = 0; q < 3; ++q) issue();
-  wait_slabs(2);
+  }
+  asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // slab 0 has landed (this wave's share)
   __syncthreads();
 
   bf16x8 fa_lo[4], fa_hi[4], fb0[k2NBT], fb1[k2NBT];
-  read_a(0, 0, fa_lo);
-  read_b(0, fb0);
+  read_a(0, 0, 0, fa_lo);
+  read_b(0, 0, fb0);
 
   f32x4v acc[k2NBV][k2NBT];
 #pragma unroll
@@ -580,48 +588,47 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
-  int step = 0;
-  // One slab (K = 32) = 32 MFMAs per wave in two halves of 16 (vocab blocks 0-3, then 4-7).  Each half
-  // is one scheduling region in which the group barriers put one LDS read (or DMA request) behind
-  // every MFMA, so that its issue hides under the MFMA's execution.
-  auto do_step = [&](bf16x8 (&fb_cur)[k2NBT], bf16x8 (&fb_nxt)[k2NBT]) {
-    __builtin_amdgcn_sched_barrier(0);
-    read_a(step, 4, fa_hi);
+  // 16 MFMAs on four vocab blocks; the group barriers then put one LDS read or DMA request behind
+  // every MFMA (or every second one), so that its issue hides under the MFMA's execution.
+  auto mfma_half = [&](int i0, bf16x8 (&fa)[4], bf16x8 (&fb)[k2NBT]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < k2NBT; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa_lo[i], fb_cur[j], acc[i][j], 0, 0, 0);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-    }
+        acc[i0 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], acc[i0 + i][j], 0, 0, 0);
+  };
+  int step = 0;
+  auto do_step = [&]() {
     __builtin_amdgcn_sched_barrier(0);
-    // Slab step+1 has landed for this wave; after the (fence-less) barrier it has for everyone, and
-    // everyone is past step-1, whose ring slot the next request overwrites.
-    wait_slabs(1);
+    read_a(step, 0, 4, fa_hi);
+    mfma_half(0, fa_lo, fb0);
+    pair_reads<2, 4>();
+    __builtin_amdgcn_sched_barrier(0);
+    read_a(step, 1, 0, fa_lo);
+    read_b(step, 1, fb1);
+    mfma_half(4, fa_hi, fb0);
+    pair_reads<2, 8>();
+    __builtin_amdgcn_sched_barrier(0);
+    read_a(step, 1, 4, fa_hi);
+    mfma_half(0, fa_lo, fb1);
+    pair_reads<2, 4>();
+    __builtin_amdgcn_sched_barrier(0);
+    // This wave has read all it needs of slab `step` and its share of slab step+1 has landed; after
+    // the (fence-less) barrier both hold for everyone.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
-    // Second half: first fragments of slab step+1 (after the last step a stale slot, unused) and the
-    // four DMA instructions of the next request.
+    // Last quarter: first fragments of slab step+1 (after the last step a stale buffer, unused) and the
+    // next request, which refills the buffer of slab `step`.  The DMA requests write LDS, so they keep
+    // their program order after the fragment reads.
     __builtin_amdgcn_sched_barrier(0);
-    read_a(step + 1, 0, fa_lo);
-    read_b(step + 1, fb_nxt);
+    read_a(step + 1, 0, 0, fa_lo);
+    read_b(step + 1, 0, fb0);
 #pragma unroll
     for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < k2NBT; ++j)
-        acc[4 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa_hi[i], fb_cur[j], acc[4 + i][j], 0, 0, 0);
-    // The DMA requests write LDS, so they keep their program order after the fragment reads.
+    mfma_half(4, fa_hi, fb1);
+    pair_reads<1, 8>();
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-    }
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM (DMA request)
     }
@@ -631,10 +638,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   };
 
   for (int vt = vt0; vt < vt1; ++vt) {
-    for (int kt = 0; kt < nk; kt += 2) {  // nk is even (H % 64 == 0): the hidden fragment sets alternate
-      do_step(fb0, fb1);
-      do_step(fb1, fb0);
-    }
+    for (int kt = 0; kt < nk; ++kt) do_step();
     const int v0 = vt * k2BV;
     fold_tile16<ENT>(acc, st, tx, tgt, v0 + wave_v * kWaveV, g, v0 + k2BV > a.V, a.V, a.scale);
 #pragma unroll
@@ -644,6 +648,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no request may outlive the workgroup's LDS
 
   write_partials16(st, tx, a.partials, t0 + wave_t * kWaveT, n_valid, split * kPartsPerSplit + wave_v,
                    sch.n_splits * kPartsPerSplit, l16, g, a.scale);
@@ -1057,10 +1062,10 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   // Measured on MI355X: the wide path wins from H = 4096 up (its exposed epilogue costs more than its
   // leaner K loop gains on short K), the DMA path below.
   if (n_tokens > kBT && H >= 4096 && H % (2 * k3BK) == 0) p.kind = kWide;
-  else if (n_tokens > kBT && H % (2 * k2BK) == 0) p.kind = kDma;
+  else if (n_tokens > kBT && H % k2BK == 0) p.kind = kDma;
   if (const char* ov = getenv("TOME_FUSED_KERNEL")) {  // tuning knob: force a path where its shape rules allow
     if (ov[0] == 'g') p.kind = kGeneric;
-    if (ov[0] == 'd' && H % (2 * k2BK) == 0) p.kind = kDma;
+    if (ov[0] == 'd' && H % k2BK == 0) p.kind = kDma;
     if (ov[0] == 'w' && H % (2 * k3BK) == 0) p.kind = kWide;
   }
   p.bt = p.kind == kGeneric ? kBT : k2BT;   // the DMA and wide paths share the 256 x 256 tile
