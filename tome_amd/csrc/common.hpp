@@ -20,6 +20,22 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
+// Plain v_max_f32 / v_max3_f32.  fmaxf() first canonicalises every operand the compiler cannot prove
+// quiet (one extra v_max per MFMA result or loaded value); the instructions themselves already return
+// the non-NaN operand, which is all the max tracking needs.
+__device__ __forceinline__ float raw_max(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+// max(x, kMaxFloor) as one v_med3_f32 (no canonicalisation, and visible to the scheduler).
+__device__ __forceinline__ float clamp_below(float x) { return __builtin_amdgcn_fmed3f(x, kMaxFloor, INFINITY); }
+__device__ __forceinline__ float raw_max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }

@@ -47,12 +47,106 @@ struct FusedPartial {  // 32 bytes per (token, part)
   int pad[3];
 };
 
+// Work decomposition: token tiles x vocab splits.  It depends on the number of valid tokens, which is
+// known on the host without a mask and only on the device with one, so it is computed by the host (and
+// passed by value) or by compact_rows_kernel (and read from the workspace header); both run the
+// same code.  Every kernel of a launch uses the same numbers.
+//
+// A workgroup owns one token tile and one contiguous range of vocab tiles.
+//   * Few token tiles (n_ttiles * 8 <= slots): as many splits as fill the chip in ONE round, rounded
+//     down - one workgroup too many would cost a whole extra round.
+//   * Many token tiles: several rounds.  The candidates 1..32 are priced as
+//         rounds * (longest vocab range + half a tile of prologue) * L2 penalty
+//     where the penalty prefers >= 8 splits: the workgroups resident on an XCD are then a block of
+//     ~4 token tiles x ~8 splits, which read 12 distinct slab streams through its L2 instead of 33
+//     (measured on MI355X: 65536 tokens, H = 4096: 1 split 1.09 PFLOP/s, 8-9 splits 1.4).
+struct FusedSchedule {
+  int n_ttiles, n_splits, n_wg, pad;
+};
+__host__ __device__ inline int64_t fused_split_cost(int n_ttiles, int n_splits, int slots, int n_vtiles) {
+  const int rounds = (n_ttiles * n_splits + slots - 1) / slots;
+  const int longest = (n_vtiles + n_splits - 1) / n_splits;
+  const int pen64 = 60 + 32 / (n_splits < 8 ? n_splits : 8);
+  return ((int64_t)rounds * (2 * longest + 1) * pen64) * 64 + n_splits;  // ties go to fewer splits
+}
+__host__ __device__ inline int fused_ttiles(int n_valid, int bt) {
+  const int t = (n_valid + bt - 1) / bt;
+  return t < 1 ? 1 : t;
+}
+__host__ __device__ inline int fused_one_round_splits(int n_ttiles, int slots, int n_vtiles) {
+  int sp = slots / n_ttiles;
+  if (sp > n_vtiles) sp = n_vtiles;
+  return sp < 1 ? 1 : sp;
+}
+constexpr int kSplitCandidates = 32;
+inline FusedSchedule fused_schedule(int n_valid, int bt, int slots, int n_vtiles) {  // host
+  FusedSchedule s;
+  s.n_ttiles = fused_ttiles(n_valid, bt);
+  s.pad = 0;
+  if (s.n_ttiles * 8 <= slots) {
+    s.n_splits = fused_one_round_splits(s.n_ttiles, slots, n_vtiles);
+  } else {
+    int64_t best = INT64_MAX;
+    for (int c = 1; c <= kSplitCandidates && c <= n_vtiles; ++c) {
+      const int64_t cost = fused_split_cost(s.n_ttiles, c, slots, n_vtiles);
+      if (cost < best) best = cost;
+    }
+    s.n_splits = (int)(best & 63);
+  }
+  s.n_wg = s.n_ttiles * s.n_splits;
+  return s;
+}
+// The same on the device, by one whole wave: lane c prices c + 1 splits.
+__device__ inline FusedSchedule fused_schedule_wave(int n_valid, int bt, int slots, int n_vtiles, int lane) {
+  FusedSchedule s;
+  s.n_ttiles = fused_ttiles(n_valid, bt);
+  s.pad = 0;
+  if (s.n_ttiles * 8 <= slots) {
+    s.n_splits = fused_one_round_splits(s.n_ttiles, slots, n_vtiles);
+  } else {
+    const int c = lane + 1;
+    int64_t cost = (c <= kSplitCandidates && c <= n_vtiles) ? fused_split_cost(s.n_ttiles, c, slots, n_vtiles) : INT64_MAX;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const int64_t o = __shfl_xor(cost, off, 64);
+      cost = o < cost ? o : cost;
+    }
+    s.n_splits = (int)(cost & 63);
+  }
+  s.n_wg = s.n_ttiles * s.n_splits;
+  return s;
+}
+
+// Workgroup id -> (token tile, vocab split).  The hardware deals consecutive workgroup ids round-robin
+// over the 8 XCDs, each with its own L2; XCD x is given the contiguous logical ids
+// [x * per, (x + 1) * per), and logical ids run over blocks of <= 8 splits, token tile by token tile,
+// so that the workgroups resident on an XCD at any time share token tiles AND vocab ranges.
+__device__ __forceinline__ bool fused_locate(const FusedSchedule& s, int bid, int& ttile, int& split) {
+  const int per = (s.n_wg + 7) >> 3;
+  const int li = bid >> 3;
+  int g = (bid & 7) * per + li;
+  if (li >= per || g >= s.n_wg) return false;  // the grid is sized for the worst case over n_valid
+  const int nb = (s.n_splits + 7) >> 3, base = s.n_splits / nb, rem = s.n_splits % nb;
+  int s0 = 0, w = base;
+  for (int sb = 0; sb < nb; ++sb) {
+    w = base + (sb < rem ? 1 : 0);
+    const int cnt = s.n_ttiles * w;
+    if (g < cnt) break;
+    g -= cnt;
+    s0 += w;
+  }
+  ttile = g / w;
+  split = s0 + g % w;
+  return true;
+}
+
 struct FusedArgs {
   const char* hidden;
   const char* weight;
   const int32_t* targets;
   const int32_t* row_index;  // compacted valid rows, or nullptr = identity
   const int32_t* n_valid;    // device scalar, or nullptr = n_tokens
+  const FusedSchedule* sched_dev;  // written by compact_rows_kernel next to n_valid, or nullptr = `sched`
   FusedPartial* partials;
   uint32_t hidden_stride_b;  // bytes
   uint32_t weight_stride_b;
@@ -63,24 +157,8 @@ struct FusedArgs {
   int n_vtiles;
   int slots;                 // workgroups that fit the chip at once (the schedule aims at one round)
   float scale;               // log2(e) / temperature
+  FusedSchedule sched;       // host-computed schedule (no mask)
 };
-
-// Work decomposition, computed on the DEVICE from the number of valid tokens (known only there when a
-// mask is given): token tiles x vocab splits, with just enough splits to fill `slots` workgroups.
-// Every kernel of a launch derives the same numbers from the same inputs.
-struct FusedSchedule {
-  int n_ttiles, n_splits, n_wg;
-};
-__host__ __device__ inline FusedSchedule fused_schedule(int n_valid, int bt, int slots, int n_vtiles) {
-  FusedSchedule s;
-  s.n_ttiles = (n_valid + bt - 1) / bt;
-  if (s.n_ttiles < 1) s.n_ttiles = 1;
-  s.n_splits = slots / s.n_ttiles;  // rounded down: one workgroup too many would cost a whole extra round
-  if (s.n_splits > n_vtiles) s.n_splits = n_vtiles;
-  if (s.n_splits < 1) s.n_splits = 1;
-  s.n_wg = s.n_ttiles * s.n_splits;
-  return s;
-}
 
 // Raw buffer descriptors: 16-byte loads addressed by a 32-bit per-lane byte offset plus a
 // uniform (scalar) offset.  A per-lane offset at or past num_bytes reads as zero, which is how
@@ -131,7 +209,7 @@ __device__ __forceinline__ void fold_tile(f32x16 (&acc)[NBV][NBT], RowStat (&st)
     for (int i = 0; i < NBV; ++i) {
       float m = acc[i][j][0];
 #pragma unroll
-      for (int e = 1; e < 16; e += 2) m = fmaxf(m, fmaxf(acc[i][j][e], e + 1 < 16 ? acc[i][j][e + 1] : acc[i][j][e]));
+      for (int e = 1; e < 16; e += 2) m = raw_max3(m, acc[i][j][e], e + 1 < 16 ? acc[i][j][e + 1] : acc[i][j][e]);
       bm[i] = m;
     }
     float cm = st[j].mx;
@@ -140,7 +218,7 @@ __device__ __forceinline__ void fold_tile(f32x16 (&acc)[NBV][NBT], RowStat (&st)
     for (int i = 0; i < NBV; ++i) {
       const bool up = bm[i] > cm;
       bi = up ? (vw0 + i * 32) : bi;  // first row of the 32-row block
-      cm = fmaxf(cm, bm[i]);
+      cm = raw_max(cm, bm[i]);
     }
     const float resc = fast_exp2((st[j].mx - cm) * scale);
     const float m = cm * scale;
@@ -155,8 +233,8 @@ __device__ __forceinline__ void fold_tile(f32x16 (&acc)[NBV][NBT], RowStat (&st)
         s0 += e0;
         s1 += e1;
         if constexpr (ENT) {
-          w0 = fmaf(fmaxf(x0, kMaxFloor) * scale, e0, w0);
-          w1 = fmaf(fmaxf(x1, kMaxFloor) * scale, e1, w1);
+          w0 = fmaf(clamp_below(x0) * scale, e0, w0);
+          w1 = fmaf(clamp_below(x1) * scale, e1, w1);
         }
       }
     st[j].mx = cm;
@@ -197,15 +275,9 @@ __global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) 
   char* ldsB = lds + kBV * kPitch;
 
   const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
-  const FusedSchedule sch = fused_schedule(n_valid, kBT, a.slots, a.n_vtiles);
-  int bid = blockIdx.x;
-  if (n_valid <= 0 || bid >= sch.n_wg) return;  // the grid is sized for the worst case over n_valid
-  // XCD-aware remap: hardware deals consecutive workgroup ids round-robin over the 8 XCDs;
-  // give each XCD a contiguous block of logical ids (= a few token tiles x all splits) so the
-  // hidden tiles it touches stay in its own L2.
-  if ((sch.n_wg & 7) == 0) bid = (bid & 7) * (sch.n_wg >> 3) + (bid >> 3);
-  const int ttile = bid / sch.n_splits;
-  const int split = bid % sch.n_splits;
+  const FusedSchedule sch = a.sched_dev ? *a.sched_dev : a.sched;
+  int ttile, split;
+  if (n_valid <= 0 || !fused_locate(sch, blockIdx.x, ttile, split)) return;
   const int t0 = ttile * kBT;
   const int vt0 = (int)((int64_t)split * a.n_vtiles / sch.n_splits);
   const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / sch.n_splits);
@@ -350,10 +422,10 @@ __device__ __forceinline__ void fold_tile16(f32x4v (&acc)[NBV][NBT], RowStat (&s
     int bi = st[j].bi;
 #pragma unroll
     for (int i = 0; i < NBV; ++i) {
-      const float bm = fmaxf(fmaxf(acc[i][j][0], acc[i][j][1]), fmaxf(acc[i][j][2], acc[i][j][3]));
+      const float bm = raw_max3(acc[i][j][0], acc[i][j][1], raw_max(acc[i][j][2], acc[i][j][3]));
       const bool up = bm > cm;
       bi = up ? (vw0 + i * 16) : bi;  // first row of the 16-row block
-      cm = fmaxf(cm, bm);
+      cm = raw_max(cm, bm);
     }
     const float resc = fast_exp2((st[j].mx - cm) * scale);
     const float m = cm * scale;
@@ -368,8 +440,8 @@ __device__ __forceinline__ void fold_tile16(f32x4v (&acc)[NBV][NBT], RowStat (&s
         s0 += e0;
         s1 += e1;
         if constexpr (ENT) {
-          w0 = fmaf(fmaxf(x0, kMaxFloor) * scale, e0, w0);
-          w1 = fmaf(fmaxf(x1, kMaxFloor) * scale, e1, w1);
+          w0 = fmaf(clamp_below(x0) * scale, e0, w0);
+          w1 = fmaf(clamp_below(x1) * scale, e1, w1);
         }
       }
     st[j].mx = cm;
@@ -465,12 +537,9 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
-  const FusedSchedule sch = fused_schedule(n_valid, k2BT, a.slots, a.n_vtiles);
-  int bid = blockIdx.x;
-  if (n_valid <= 0 || bid >= sch.n_wg) return;  // the grid is sized for the worst case over n_valid
-  if ((sch.n_wg & 7) == 0) bid = (bid & 7) * (sch.n_wg >> 3) + (bid >> 3);  // contiguous logical ids per XCD
-  const int ttile = bid / sch.n_splits;
-  const int split = bid % sch.n_splits;
+  const FusedSchedule sch = a.sched_dev ? *a.sched_dev : a.sched;
+  int ttile, split;
+  if (n_valid <= 0 || !fused_locate(sch, blockIdx.x, ttile, split)) return;
   const int t0 = ttile * k2BT;
   const int vt0 = (int)((int64_t)split * a.n_vtiles / sch.n_splits);
   const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / sch.n_splits);
@@ -654,234 +723,6 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
                    sch.n_splits * kPartsPerSplit, l16, g, a.scale);
 }
 
-// ===============================================================================================
-// Wide path (H % 128 == 0): 256 lanes = one wave per SIMD, 256 x 256 tile, 128 x 128 wave tiles.
-//
-//   * 4 waves as 2 (vocab) x 2 (token).  A wave owns 4 x 4 accumulator blocks (256 registers, which
-//     the compiler keeps in AGPRs), so each fragment read from LDS feeds four MFMAs instead of
-//     two or four of the 2-waves-per-SIMD layouts: a third fewer LDS bytes per MFMA.
-//   * K slabs are 64 wide (128-byte rows, whole cache lines per request).  With one wave per SIMD
-//     the other 256 VGPRs are free, and two of the slabs in flight live there: slab s+2 is loaded
-//     global -> registers during step s, written registers -> LDS during step s+1 and multiplied
-//     in step s+2, so a load has more than a full step (64 MFMAs per wave) to arrive.  LDS holds
-//     two 64 KB slabs, XOR-swizzled like the DMA path (chunk c of row r at c ^ ((r >> 1) & 7)).
-//   * Two fence-less barriers per step, neither followed by a dependent LDS read: B1 (after
-//     sub-step 0) says everybody is done with slab s-1, whose slot the writes of sub-steps 1-2
-//     then refill; B2 (after sub-step 2) publishes slab s+1 before sub-step 3 prefetches its first
-//     fragments.  The MFMA stream runs through step and vocab-tile boundaries without a bubble.
-// ===============================================================================================
-constexpr int k3WG = 256;
-constexpr int k3BV = 256, k3BT = 256, k3BK = 64;
-constexpr int k3WaveV = 128, k3WaveT = 128;
-constexpr int k3NBV = k3WaveV / 32, k3NBT = k3WaveT / 32;
-constexpr int k3RowBytes = k3BK * 2;                      // 128
-constexpr int k3SlabBytes = (k3BV + k3BT) * k3RowBytes;   // 65536
-constexpr int k3LdsTotal = 2 * k3SlabBytes;
-constexpr int k3Loads = k3BV * 8 / k3WG;                  // 16-byte loads per lane, operand and slab (8)
-
-template <bool ENT>
-__global__ __launch_bounds__(k3WG) void fused_lmhead_wide_kernel(FusedArgs a) {
-  extern __shared__ __attribute__((aligned(1024))) char smem[];
-
-  const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
-  const FusedSchedule sch = fused_schedule(n_valid, k3BT, a.slots, a.n_vtiles);
-  int bid = blockIdx.x;
-  if (n_valid <= 0 || bid >= sch.n_wg) return;  // the grid is sized for the worst case over n_valid
-  if ((sch.n_wg & 7) == 0) bid = (bid & 7) * (sch.n_wg >> 3) + (bid >> 3);  // contiguous logical ids per XCD
-  const int ttile = bid / sch.n_splits;
-  const int split = bid % sch.n_splits;
-  const int t0 = ttile * k3BT;
-  const int vt0 = (int)((int64_t)split * a.n_vtiles / sch.n_splits);
-  const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / sch.n_splits);
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wave_v = wave & 1, wave_t = wave >> 1;
-  const int l32 = lane & 31, lh = lane >> 5;
-
-  // ---- staging assignment: load j of wave w covers tile rows (j*4 + w)*8 .. +7 of an operand ------
-  const int dr = lane >> 3;                                     // row inside the 8-row group
-  const int dc = (lane & 7) ^ (((wave & 1) << 2) | (dr >> 1));  // global chunk: position ^ ((row >> 1) & 7)
-  const __amdgpu_buffer_rsrc_t rsrcB = make_rsrc(a.hidden, a.hidden_bytes);
-  uint32_t aoff[k3Loads], boff[k3Loads];
-#pragma unroll
-  for (int j = 0; j < k3Loads; ++j) {
-    const int r = (j * 4 + wave) * 8 + dr;
-    aoff[j] = (uint32_t)r * a.weight_stride_b + dc * 16;
-    int p = t0 + r;
-    p = p < n_valid ? p : n_valid - 1;
-    const int tok = a.row_index ? a.row_index[p] : p;
-    boff[j] = (uint32_t)tok * a.hidden_stride_b + dc * 16;
-  }
-  const int st_off = wave * 1024 + lane * 16;  // where this lane's 16 bytes of load j land: + j * 4096
-
-  RowStat st[k3NBT];
-  float tx[k3NBT];
-  int tgt[k3NBT];
-#pragma unroll
-  for (int bt = 0; bt < k3NBT; ++bt) {
-    st[bt] = stat_identity();
-    tx[bt] = -INFINITY;
-    const int p = t0 + wave_t * k3WaveT + bt * 32 + l32;
-    int t = -1;
-    if (p < n_valid) t = a.targets[a.row_index ? a.row_index[p] : p];
-    tgt[bt] = (t >= 0 && t < a.V) ? t : -1;
-  }
-
-  // ---- fragment read offsets inside a slab (swizzled) --------------------------------------------
-  const int x7 = (l32 >> 1) & 7;
-  int swz[4];
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) swz[ks] = ((ks * 2 + lh) ^ x7) * 16;
-  const int rdA = (wave_v * k3WaveV + l32) * k3RowBytes;
-  const int rdB = k3BV * k3RowBytes + (wave_t * k3WaveT + l32) * k3RowBytes;
-
-  const int nk = a.H / k3BK;
-
-  // The load stream runs two slabs ahead of the multiply; it keeps its own (tile, slab) position.
-  int l_kt = 0, l_vt = vt0;
-  __amdgpu_buffer_rsrc_t rsrcA =
-      make_rsrc(a.weight + (int64_t)l_vt * k3BV * a.weight_stride_b, (uint32_t)(a.V - l_vt * k3BV) * a.weight_stride_b);
-  // Two register sets for W (a set is written to LDS one step after it was loaded), one for hidden
-  // (its write, sub-step 2, precedes its next load, sub-step 3).  The sets are separate arrays picked
-  // at compile time: a run-time index would push them into private memory.
-  u32x4 ra0[k3Loads], ra1[k3Loads], rb[k3Loads];
-  auto load_w = [&](u32x4 (&ra)[k3Loads]) {  // W rows of slab (l_vt, l_kt)
-    const uint32_t koff = (uint32_t)l_kt * k3RowBytes;
-#pragma unroll
-    for (int j = 0; j < k3Loads; ++j) ra[j] = ld16(rsrcA, aoff[j], koff);
-  };
-  auto load_h = [&]() {  // hidden rows of the same slab
-    const uint32_t koff = (uint32_t)l_kt * k3RowBytes;
-#pragma unroll
-    for (int j = 0; j < k3Loads; ++j) rb[j] = ld16(rsrcB, boff[j], koff);
-  };
-  auto load_advance = [&]() {  // past the last slab the stream stays on it: the loads below are issued
-    if (l_vt == vt1 - 1 && l_kt == nk - 1) return;  // unconditionally, and re-reading it is harmless
-    if (++l_kt == nk) {
-      l_kt = 0;
-      ++l_vt;
-      rsrcA = make_rsrc(a.weight + (int64_t)l_vt * k3BV * a.weight_stride_b,
-                        (uint32_t)(a.V - l_vt * k3BV) * a.weight_stride_b);
-    }
-  };
-  auto write_w = [&](const u32x4 (&ra)[k3Loads], int slot) {
-    char* dst = smem + slot * k3SlabBytes + st_off;
-#pragma unroll
-    for (int j = 0; j < k3Loads; ++j) *reinterpret_cast<u32x4*>(dst + j * 4096) = ra[j];
-  };
-  auto write_h = [&](int slot) {
-    char* dst = smem + slot * k3SlabBytes + st_off + k3BV * k3RowBytes;
-#pragma unroll
-    for (int j = 0; j < k3Loads; ++j) *reinterpret_cast<u32x4*>(dst + j * 4096) = rb[j];
-  };
-  auto read_frags = [&](int slot, int ks, bf16x8 (&fa)[k3NBV], bf16x8 (&fb)[k3NBT]) {
-    const char* slab = smem + slot * k3SlabBytes;
-#pragma unroll
-    for (int i = 0; i < k3NBV; ++i)
-      fa[i] = *reinterpret_cast<const bf16x8*>(slab + rdA + i * 32 * k3RowBytes + swz[ks]);
-#pragma unroll
-    for (int j = 0; j < k3NBT; ++j)
-      fb[j] = *reinterpret_cast<const bf16x8*>(slab + rdB + j * 32 * k3RowBytes + swz[ks]);
-  };
-
-  // ---- prologue: slab 0 through registers into LDS slot 0, slab 1 into register set 1 --------------
-  load_w(ra0);
-  load_h();
-  load_advance();
-  write_w(ra0, 0);
-  write_h(0);
-  load_w(ra1);
-  load_h();
-  load_advance();
-  __syncthreads();
-
-  bf16x8 fa0[k3NBV], fb0[k3NBT], fa1[k3NBV], fb1[k3NBT];
-  read_frags(0, 0, fa0, fb0);
-
-  f32x16 acc[k3NBV][k3NBT];
-#pragma unroll
-  for (int i = 0; i < k3NBV; ++i)
-#pragma unroll
-    for (int j = 0; j < k3NBT; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-#define TOME_MFMA_BLOCK(FA, FB)                                                                    \
-  _Pragma("unroll") for (int i = 0; i < k3NBV; ++i) _Pragma("unroll") for (int j = 0; j < k3NBT; ++j) \
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FA[i], FB[j], acc[i][j], 0, 0, 0)
-
-  // One K slab s.  ra_cur is the W register set that held slab s (free now, receives slab s+2),
-  // ra_nxt holds slab s+1; `cur` is the LDS slot of slab s.
-  auto do_step = [&](u32x4 (&ra_cur)[k3Loads], u32x4 (&ra_nxt)[k3Loads], int cur) {
-    const int nxt = cur ^ 1;
-    // Every load and LDS write below is issued on every step, also when the slab it belongs to does
-    // not exist any more (then it moves stale data into a slot nobody reads): under a branch the
-    // wait-count insertion must assume the newest loads may be absent and drains them all.
-    // Each sub-step is one scheduling region: 16 MFMAs, 8 fragment reads for the next sub-step and 8
-    // staging instructions.  The group barriers ask for one memory instruction behind every MFMA, so
-    // that its issue time hides under the 32 cycles the MFMA executes; issued as a clump they would
-    // leave the matrix pipe idle (one wave per SIMD: nobody else fills the gap).
-#define TOME_INTERLEAVE(MEM_MASK)                                    \
-  _Pragma("unroll") for (int q = 0; q < 8; ++q) {                    \
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* MFMA */    \
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); /* DS read */ \
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               \
-    __builtin_amdgcn_sched_group_barrier(MEM_MASK, 1, 0);            \
-  }
-    // sub-step 0: fragments of k1; W rows of slab step+2
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(cur, 1, fa1, fb1);
-    load_w(ra_cur);
-    TOME_MFMA_BLOCK(fa0, fb0);
-    TOME_INTERLEAVE(0x020)
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_barrier();  // B1: nobody reads slab step-1 any more; its slot may be refilled
-    // sub-step 1: fragments of k2; W half of slab step+1 goes registers -> LDS
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(cur, 2, fa0, fb0);
-    write_w(ra_nxt, nxt);
-    TOME_MFMA_BLOCK(fa1, fb1);
-    TOME_INTERLEAVE(0x200)
-    // sub-step 2: fragments of k3; hidden half of slab step+1
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(cur, 3, fa1, fb1);
-    write_h(nxt);
-    TOME_MFMA_BLOCK(fa0, fb0);
-    TOME_INTERLEAVE(0x200)
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's LDS writes are done
-    __builtin_amdgcn_s_barrier();                        // B2: slab step+1 is complete and visible
-    // sub-step 3: first fragments of slab step+1 (a stale slot after the last step, unused);
-    // hidden rows of slab step+2
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(nxt, 0, fa0, fb0);
-    load_h();
-    load_advance();
-    TOME_MFMA_BLOCK(fa1, fb1);
-    TOME_INTERLEAVE(0x020)
-    __builtin_amdgcn_sched_barrier(0);
-#undef TOME_INTERLEAVE
-  };
-  for (int vt = vt0; vt < vt1; ++vt) {
-    for (int kt = 0; kt < nk; kt += 2) {  // nk is even (H % 128 == 0): slab parity == kt parity
-      do_step(ra0, ra1, 0);
-      do_step(ra1, ra0, 1);
-    }
-    const int v0 = vt * k3BV;
-    fold_tile<ENT>(acc, st, tx, tgt, v0 + wave_v * k3WaveV, lh, v0 + k3BV > a.V, a.V, a.scale);
-#pragma unroll
-    for (int i = 0; i < k3NBV; ++i)
-#pragma unroll
-      for (int j = 0; j < k3NBT; ++j)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-  }
-#undef TOME_MFMA_BLOCK
-
-  write_partials(st, tx, a.partials, t0 + wave_t * k3WaveT, n_valid, split * kPartsPerSplit + wave_v,
-                 sch.n_splits * kPartsPerSplit, l32, lh, a.scale);
-}
-
 // ---- compaction of valid rows ----------------------------------------------------------------
 // One workgroup: row_index[0 .. n_valid) = ascending indices of rows with row_valid != 0.
 // Outputs of masked rows are zeroed here.
@@ -895,6 +736,7 @@ struct CompactArgs {
   float* out3;
   int32_t* out_argmax;
   int n;
+  int bt, slots, n_vtiles;  // inputs of the schedule, which this kernel derives from n_valid
 };
 
 __global__ __launch_bounds__(1024) void compact_rows_kernel(CompactArgs a) {
@@ -927,6 +769,11 @@ __global__ __launch_bounds__(1024) void compact_rows_kernel(CompactArgs a) {
     }
   }
   if (tid == 1023) *a.n_valid = base + inc;
+  if (wave == 15) {  // the last wave knows the total: it also fixes the work decomposition
+    const int total = __shfl(base + inc, 63, 64);
+    const FusedSchedule sch = fused_schedule_wave(total, a.bt, a.slots, a.n_vtiles, lane);
+    if (lane == 0) *reinterpret_cast<FusedSchedule*>(a.n_valid + 4) = sch;
+  }
 }
 
 // ---- combine -----------------------------------------------------------------------------------
@@ -948,7 +795,8 @@ struct CombineArgs {
   int H;
   int V;
   int n_tokens;
-  int bt, slots, n_vtiles;  // inputs of fused_schedule, to find the number of parts per token
+  const FusedSchedule* sched_dev;  // as in FusedArgs
+  FusedSchedule sched;
   float scale;
 };
 
@@ -1013,7 +861,7 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
   const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
   if (p >= n_valid) return;
   const int tok = a.row_index ? a.row_index[p] : p;
-  const int n_parts = fused_schedule(n_valid, a.bt, a.slots, a.n_vtiles).n_splits * kPartsPerSplit;
+  const int n_parts = (a.sched_dev ? a.sched_dev->n_splits : a.sched.n_splits) * kPartsPerSplit;
   RowStat st;
   float tx;
   combine_one(a.partials + (int64_t)p * n_parts, n_parts, lane, a.scale, st, tx);
@@ -1044,10 +892,10 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
 }
 
 // ---- host side -----------------------------------------------------------------------------------
-// The wide and DMA kernels need whole 64- / 32-wide K slabs and pay for 256-token tiles; short
-// batches and ragged H go to the generic kernel.
+// The DMA kernel needs whole 64-wide K slabs and pays for 256-token tiles; short batches and ragged H
+// go to the generic kernel.
 
-enum FusedKind { kGeneric = 0, kDma = 1, kWide = 2 };
+enum FusedKind { kGeneric = 0, kDma = 1 };
 
 struct FusedPlan {
   FusedKind kind;
@@ -1059,16 +907,12 @@ struct FusedPlan {
 static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   FusedPlan p;
   p.kind = kGeneric;
-  // Measured on MI355X: the wide path wins from H = 4096 up (its exposed epilogue costs more than its
-  // leaner K loop gains on short K), the DMA path below.
-  if (n_tokens > kBT && H >= 4096 && H % (2 * k3BK) == 0) p.kind = kWide;
-  else if (n_tokens > kBT && H % k2BK == 0) p.kind = kDma;
+  if (n_tokens > kBT && H % k2BK == 0) p.kind = kDma;
   if (const char* ov = getenv("TOME_FUSED_KERNEL")) {  // tuning knob: force a path where its shape rules allow
     if (ov[0] == 'g') p.kind = kGeneric;
     if (ov[0] == 'd' && H % k2BK == 0) p.kind = kDma;
-    if (ov[0] == 'w' && H % (2 * k3BK) == 0) p.kind = kWide;
   }
-  p.bt = p.kind == kGeneric ? kBT : k2BT;   // the DMA and wide paths share the 256 x 256 tile
+  p.bt = p.kind == kGeneric ? kBT : k2BT;   // the DMA path has a 256 x 256 tile
   p.bv = p.kind == kGeneric ? kBV : k2BV;
   p.slots = p.kind == kGeneric ? 512 : 256;  // resident workgroups on 256 CUs: 2 per CU, or 1 (128 KB LDS)
   p.n_vtiles = (int)((V + p.bv - 1) / p.bv);
@@ -1077,7 +921,8 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   const int tt_max = (int)((n_tokens + p.bt - 1) / p.bt);
   for (int tt = 1; tt <= tt_max; ++tt) {  // the schedule depends on n_valid only through its tile count
     const FusedSchedule s = fused_schedule(tt * p.bt, p.bt, p.slots, p.n_vtiles);
-    if (s.n_wg > p.grid) p.grid = s.n_wg;
+    const int padded = 8 * ((s.n_wg + 7) / 8);  // fused_locate deals whole rows of 8 workgroup ids
+    if (padded > p.grid) p.grid = padded;
     const size_t rec = (size_t)tt * p.bt * s.n_splits * kPartsPerSplit;
     if (rec > p.max_records) p.max_records = rec;
   }
@@ -1105,12 +950,9 @@ static void launch_main(const FusedArgs& a, FusedKind kind, int grid, hipStream_
   static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
   if (!attr_set) {
     allow_big_lds(&fused_lmhead_dma_kernel<ENT>, k2LdsTotal);
-    allow_big_lds(&fused_lmhead_wide_kernel<ENT>, k3LdsTotal);
     attr_set = true;
   }
-  if (kind == kWide) {
-    hipLaunchKernelGGL(fused_lmhead_wide_kernel<ENT>, dim3((unsigned)grid), dim3(k3WG), k3LdsTotal, stream, a);
-  } else if (kind == kDma) {
+  if (kind == kDma) {
     hipLaunchKernelGGL(fused_lmhead_dma_kernel<ENT>, dim3((unsigned)grid), dim3(k2WG), k2LdsTotal, stream, a);
   } else {
     hipLaunchKernelGGL(fused_lmhead_kernel<ENT>, dim3((unsigned)grid), dim3(kFusedWG), 0, stream, a);
@@ -1123,15 +965,18 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w
                                float* out_entropy, int32_t* out_argmax, float* out_ref_lp, float* out_k3,
                                void* workspace, hipStream_t stream) {
   char* ws = static_cast<char*>(workspace);
+  const FusedPlan plan = fused_plan(n_tokens, H, V);
   int32_t* n_valid = nullptr;
   int32_t* row_index = nullptr;
   if (row_valid) {
     n_valid = reinterpret_cast<int32_t*>(ws);
     row_index = reinterpret_cast<int32_t*>(ws + off_index());
-    CompactArgs c{row_valid, row_index, n_valid, out_lp, out_lse, out_entropy, out_ref_lp, out_argmax, (int)n_tokens};
+    CompactArgs c{row_valid, row_index, n_valid, out_lp, out_lse, out_entropy, out_ref_lp, out_argmax, (int)n_tokens,
+                  plan.bt, plan.slots, plan.n_vtiles};
     hipLaunchKernelGGL(compact_rows_kernel, dim3(1), dim3(1024), 0, stream, c);
     if (out_k3) {
-      CompactArgs c2{row_valid, row_index, n_valid, out_k3, nullptr, nullptr, nullptr, nullptr, (int)n_tokens};
+      CompactArgs c2{row_valid, row_index, n_valid, out_k3, nullptr, nullptr, nullptr, nullptr, (int)n_tokens,
+                     plan.bt, plan.slots, plan.n_vtiles};
       hipLaunchKernelGGL(compact_rows_kernel, dim3(1), dim3(1024), 0, stream, c2);
     }
     hipError_t e = hipGetLastError();
@@ -1148,9 +993,11 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w
   a.n_tokens = (int)n_tokens;
   a.H = (int)H;
   a.V = (int)V;
-  const FusedPlan plan = fused_plan(n_tokens, H, V);
   a.n_vtiles = plan.n_vtiles;
   a.slots = plan.slots;
+  // Workspace header: [0] n_valid, [16..32) the schedule derived from it on the device.
+  a.sched_dev = row_valid ? reinterpret_cast<const FusedSchedule*>(n_valid + 4) : nullptr;
+  a.sched = fused_schedule((int)n_tokens, plan.bt, plan.slots, plan.n_vtiles);
   a.scale = kLog2e / temperature;
   FusedPartial* p0 = reinterpret_cast<FusedPartial*>(ws + off_partials(n_tokens));
   FusedPartial* p1 = reinterpret_cast<FusedPartial*>(ws + off_partials(n_tokens) + partial_bytes(n_tokens, H, V));
@@ -1185,9 +1032,8 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w
   c.H = a.H;
   c.V = a.V;
   c.n_tokens = (int)n_tokens;
-  c.bt = plan.bt;
-  c.slots = plan.slots;
-  c.n_vtiles = plan.n_vtiles;
+  c.sched_dev = a.sched_dev;
+  c.sched = a.sched;
   c.scale = a.scale;
   hipLaunchKernelGGL(fused_combine_kernel, dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, stream, c);
   return hipGetLastError();
