@@ -93,6 +93,24 @@ int tome_fused_lmhead_logprob(const void* hidden, const void* weight, int64_t n_
                               float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
                               void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- Final RMSNorm + lm_head + log-softmax ------------------------------------------
+ * The same with the model's last normalisation folded in: replaces
+ *   x = self.norm(x); logits = x @ embed_tokens.weight.T      mlx-impl/model.py:536-538
+ *   (RMSNorm = mx.fast.rms_norm(x, weight, eps),               mlx-impl/model.py:336-343)
+ * followed by local_compute_logprobs (mlx-impl/node.py:400-404).  `hidden` holds the
+ * PRE-norm states of the last decoder layer, `norm_weight` is bf16 [H].  Only rows with
+ * row_valid != 0 are normalised - y = w * bf16(x * rsqrt(mean(x^2) + eps)), statistics in
+ * fp32, as MLX computes it - into the workspace and then multiplied, so the prompt and pad
+ * rows that node.py:443-449 computes and discards cost nothing here.
+ */
+size_t tome_norm_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V);
+int tome_norm_lmhead_logprob(const void* hidden, const void* norm_weight, float norm_eps,
+                             const void* weight, int64_t n_tokens, int64_t H, int64_t V,
+                             int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
+                             const int32_t* row_valid, float temperature, float* out_lp,
+                             float* out_lse, float* out_entropy, int32_t* out_argmax,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- GRPO policy + reference dual pass --------------------------------------------
  * Two lm_head weight sets over the same hidden states (policy = reference + LoRA merge,
  * mlx-impl/node.py:102-164).  Emits per token

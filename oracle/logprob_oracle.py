@@ -43,6 +43,13 @@ Pinning (tests/test_oracle.py):
                             vs logits - logsumexp on bf16 [1,151936]) and the
                             tail cases of model.py:17-20,34-36.
   local_compute_logprobs_f32  agreement with logprob_rows within 1e-5.
+  rms_norm64 / rms_norm_bf16  the published definition of mx.fast.rms_norm
+                            (MLX, not vendored): closed forms (w = 1 -> unit RMS,
+                            x -> c x leaves y unchanged as eps -> 0, constant row
+                            -> sign(x) w), torch.nn.functional.rms_norm in float64
+                            as an independent library routine, brute force with
+                            math.fsum.  The order of MLX's two bf16 roundings
+                            (normalise, round, scale, round): parity unpinned.
   process_ref_logprobs_batched  known-answer tests on a stub model
                             (alignment, empty completion, temperature 0,
                             chunking, padding id 0) and the length contract of
@@ -59,6 +66,7 @@ __all__ = [
     "bf16_round", "bf16_to_f32", "to_f64", "lse_rows", "logprob_rows", "entropy_rows",
     "argmax_rows", "k3", "lmhead_logits64", "lmhead_stats", "full_log_softmax64",
     "local_compute_logprobs_f32", "fused_log_softmax_f32", "process_ref_logprobs_batched",
+    "rms_norm64", "rms_norm_bf16",
 ]
 
 
@@ -150,6 +158,26 @@ def lmhead_logits64(hidden: np.ndarray, weight: np.ndarray) -> np.ndarray:
     weight is [V, H] row-major as in model.py:538 (x @ embed_tokens.weight.T).
     """
     return to_f64(hidden) @ to_f64(weight).T
+
+
+def rms_norm64(x: np.ndarray, weight: np.ndarray, eps: float = 1e-6) -> np.ndarray:
+    """y = x * rsqrt(mean(x^2, -1) + eps) * w in fp64 on exactly-upcast inputs: RMSNorm.__call__ =
+    mx.fast.rms_norm(x, self.weight, self.eps) (mlx-impl/model.py:336-343), applied to the last
+    hidden states at model.py:536."""
+    x64, w64 = to_f64(x), to_f64(weight)
+    inv = 1.0 / np.sqrt((x64 * x64).mean(axis=-1, keepdims=True) + float(eps))
+    return x64 * inv * w64
+
+
+def rms_norm_bf16(x: np.ndarray, weight: np.ndarray, eps: float = 1e-6) -> np.ndarray:
+    """The same with MLX's storage roundings, bf16 bit patterns in and out: statistics in fp32, the
+    normalised value rounded to bf16, then multiplied by the bf16 weight and rounded again (the
+    published rms_norm kernel of MLX; model.py:343 passes bf16 activations and weights)."""
+    x32, w32 = bf16_to_f32(x), bf16_to_f32(weight)
+    ms = (x32.astype(np.float64) ** 2).mean(axis=-1, keepdims=True)
+    inv = (1.0 / np.sqrt(ms + float(eps))).astype(np.float32)
+    t = bf16_to_f32(bf16_round(x32 * inv))
+    return bf16_round(w32 * t)
 
 
 def lmhead_stats(hidden: np.ndarray, weight: np.ndarray, targets: np.ndarray,

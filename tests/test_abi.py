@@ -55,6 +55,8 @@ def test_workspace_queries():
     one = lib.tome_fused_lmhead_logprob_workspace(4096, 1024, 151936)
     two = lib.tome_grpo_dual_workspace(4096, 1024, 151936)
     assert 0 < one < two and one % 256 == 0
+    normed = lib.tome_norm_lmhead_logprob_workspace(4096, 1024, 151936)
+    assert normed >= one + 4096 * 1024 * 2 and normed % 256 == 0      # room for the normalised rows
 
 
 def test_argument_checks_run_on_host():
@@ -80,6 +82,10 @@ def test_argument_checks_run_on_host():
     assert fused(h=None) == -1 and fused(n=0) == 0
     assert fused(n=1 << 20, H=4096, hs=4096, ws=4096) == -3          # > 4 GiB of hidden
     assert fused() == -4                                             # workspace missing
+    norm = lambda **k: lib.tome_norm_lmhead_logprob(P, k.get("nw", P), k.get("eps", 1e-6), P, 8, k.get("H", 64), 100, 64, 64,
+                                                    P, None, 1.0, P, None, None, None, None, 0, None)
+    assert norm(nw=None) == -1 and norm(nw=P + 4) == -6 and norm(eps=-1.0) == -3 and norm(eps=float("nan")) == -3
+    assert norm(H=0) == -3 and norm() == -4
     dual = lib.tome_grpo_dual(P, P, None, 8, 64, 100, 64, 64, P, None, 1.0, P, P, P, P, None, 0, None)
     assert dual == -1
 

@@ -235,3 +235,30 @@ def test_fused_every_partial_is_written(dev, kind, n, frac_valid, monkeypatch):
     ref = torch.logsumexp(h.float() @ w.float().T, dim=-1).cpu().numpy()
     np.testing.assert_allclose(got_lse[m], ref[m], atol=TOL, rtol=0)
     assert (got_lp[~m] == 0).all()
+
+
+@pytest.mark.parametrize("n,H,V,masked", [(40, 64, 700, False), (300, 256, 3000, True), (1500, 1024, 5000, True)])
+def test_norm_lmhead_matches_oracle(dev, n, H, V, masked):
+    """Final RMSNorm folded in front of the lm_head (mlx-impl/model.py:536-538): rows are normalised as the
+    oracle's bf16 restatement does, then scored; masked rows are neither normalised nor multiplied."""
+    rng = np.random.default_rng(n + H)
+    h, w, t = _inputs(dev, n, H, V, seed=n + 1, h_scale=4.0, w_scale=0.2)
+    h = (h.float() * torch.linspace(0.2, 3.0, n, device=dev)[:, None]).to(torch.bfloat16)   # rows of very different norms
+    gamma = torch.from_numpy((1.0 + 0.2 * rng.standard_normal(H)).astype(np.float32)).to(dev).to(torch.bfloat16)
+    valid = (rng.random(n) < 0.6).astype(np.int32) if masked else np.ones(n, np.int32)
+    r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 0.9, want_lse=True, want_entropy=True, want_argmax=True,
+                                       row_valid=torch.from_numpy(valid).to(dev) if masked else None,
+                                       norm_weight=gamma, norm_eps=1e-6)
+    normed = oracle.rms_norm_bf16(bf16_bits_of(h), bf16_bits_of(gamma), 1e-6)
+    want = oracle.lmhead_stats(normed, bf16_bits_of(w), t, 0.9)
+    m = valid.astype(bool)
+    # 2e-3 of the fused path + rare one-ulp flips of a normalised value (fp32 statistics summed in another order)
+    np.testing.assert_allclose(r.lp.cpu().numpy()[m], want["lp"][m], atol=4e-3, rtol=0)
+    np.testing.assert_allclose(r.lse.cpu().numpy()[m], want["lse"][m], atol=4e-3, rtol=0)
+    np.testing.assert_allclose(r.entropy.cpu().numpy()[m], want["entropy"][m], atol=4e-3, rtol=0)
+    clear = m & ((want["top1"] - want["top2"]) > 1e-2)
+    np.testing.assert_array_equal(r.argmax.cpu().numpy()[clear], want["argmax"][clear])
+    assert (r.lp.cpu().numpy()[~m] == 0).all()
+    # the norm must really have been applied: without it the answer is far away
+    raw = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 0.9).lp.cpu().numpy()
+    assert np.abs(raw[m] - want["lp"][m]).max() > 0.1

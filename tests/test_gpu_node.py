@@ -81,6 +81,42 @@ def test_entry_hidden_state_mode_scores_only_completion_rows(dev):
             np.testing.assert_allclose(c.ref_log_probs, cw.ref_log_probs, atol=2e-3, rtol=0)
 
 
+def test_entry_prenorm_mode_applies_the_final_norm_to_completion_rows(dev):
+    """Pre-norm mode: the model returns the states BEFORE the last RMSNorm (model.py:536); norm, lm_head and
+    log-softmax all run on completion rows only."""
+    rng = np.random.default_rng(3)
+    H = 128
+    emb = oracle.bf16_round((rng.standard_normal((V_STUB, H)) * 0.5).astype(np.float32))
+    gamma = oracle.bf16_round((1.0 + 0.2 * rng.standard_normal(H)).astype(np.float32))
+    to_t = lambda bits: torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16).to(dev)
+
+    def prenorm_np(full_ids):  # toy decoder output with a position-dependent scale, so the norm matters
+        e = oracle.bf16_to_f32(emb)[full_ids.astype(np.int64)]
+        pos = np.arange(full_ids.shape[1])[None, :, None]
+        return oracle.bf16_round((e * (1.0 + 0.5 * pos) + np.roll(e, 3, -1)).astype(np.float32))
+
+    def model(full_ids, cache=None):
+        return to_t(prenorm_np(full_ids.cpu().numpy())), None
+
+    def np_model(full_ids):
+        normed = oracle.rms_norm_bf16(prenorm_np(full_ids).reshape(-1, H), gamma, 1e-6)
+        return oracle.lmhead_logits64(normed, emb).reshape(*full_ids.shape, V_STUB).astype(np.float32)
+
+    prompts, results = make_batch(seed=5, n_prompts=3, G=2)
+    want = copy.deepcopy(results)
+    oracle.process_ref_logprobs_batched(prompts, want, 2, 1.1, reference_model=np_model)
+    svc = tome_amd.RefLogprobServicer(model, device=dev, lm_head_weight=to_t(emb), final_norm_weight=to_t(gamma), norm_eps=1e-6)
+    svc.process_ref_logprobs_batched(prompts, results, 2, 1.1)
+    for r, w in zip(results, want):
+        for c, cw in zip(r.completions, w.completions):
+            assert len(c.ref_log_probs) == len(c.tokens)
+            # a bf16 rounding of a normalised value may flip where the fp32 statistics differ in the last
+            # place: 2e-3 of the fused path plus the effect of a few one-ulp flips
+            np.testing.assert_allclose(c.ref_log_probs, cw.ref_log_probs, atol=4e-3, rtol=0)
+    with pytest.raises(ValueError):
+        tome_amd.RefLogprobServicer(model, device=dev, final_norm_weight=to_t(gamma))
+
+
 # ---- golden vectors through the C ABI ------------------------------------------------------------------
 @pytest.mark.parametrize("name", ["s0", "s1", "s2"])
 def test_golden_small(dev, name):

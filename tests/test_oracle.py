@@ -210,3 +210,46 @@ def test_local_compute_logprobs_restatement_divides_by_temp():
     # bf16 input is upcast exactly first (node.py:401)
     b = oracle.bf16_round(x)
     np.testing.assert_allclose(oracle.local_compute_logprobs_f32(b, t, 0.7), oracle.logprob_rows(b, t, 0.7), atol=1e-5)
+
+
+# ---- final RMSNorm (model.py:336-343, :536) -------------------------------------------------------
+def test_rms_norm_closed_forms_and_library():
+    import torch
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((5, 96)) * 3.0
+    w = rng.standard_normal(96)
+    y = oracle.rms_norm64(x, w, 1e-6)
+    # independent library routine, float64
+    ref = torch.nn.functional.rms_norm(torch.from_numpy(x), (96,), torch.from_numpy(w), 1e-6).numpy()
+    np.testing.assert_allclose(y, ref, rtol=1e-12, atol=1e-12)
+    # brute force with exact summation: a dropped eps, a sum instead of a mean or sqrt instead of rsqrt fails
+    for r in range(5):
+        ms = math.fsum(v * v for v in x[r]) / 96
+        want = [x[r, j] / math.sqrt(ms + 1e-6) * w[j] for j in range(96)]
+        np.testing.assert_allclose(y[r], want, rtol=1e-12)
+    # closed forms: unit RMS with w = 1; scale invariance as eps -> 0; constant row -> sign(x) * w
+    y1 = oracle.rms_norm64(x, np.ones(96), 0.0)
+    np.testing.assert_allclose(np.sqrt((y1 * y1).mean(-1)), 1.0, rtol=1e-12)
+    np.testing.assert_allclose(oracle.rms_norm64(7.5 * x, w, 0.0), oracle.rms_norm64(x, w, 0.0), rtol=1e-12)
+    np.testing.assert_allclose(oracle.rms_norm64(np.full((1, 8), -2.0), np.arange(8.0), 0.0), -np.arange(8.0)[None], rtol=1e-12)
+    # eps matters for a tiny row: y = x / sqrt(x^2 + eps)
+    np.testing.assert_allclose(oracle.rms_norm64(np.full((1, 4), 1e-3), np.ones(4), 1e-6), 1e-3 / math.sqrt(2e-6), rtol=1e-12)
+
+
+def test_rms_norm_bf16_is_the_closed_form_within_two_roundings():
+    import torch
+    rng = np.random.default_rng(12)
+    xb = oracle.bf16_round((rng.standard_normal((64, 256)) * 2.0).astype(np.float32))
+    wb = oracle.bf16_round((1.0 + 0.1 * rng.standard_normal(256)).astype(np.float32))
+    yb = oracle.rms_norm_bf16(xb, wb, 1e-6)
+    assert yb.dtype == np.uint16 and yb.shape == xb.shape
+    y64 = oracle.rms_norm64(xb, wb, 1e-6)
+    got = oracle.to_f64(yb)
+    # two bf16 roundings of 2^-8 relative each (+ tiny slack)
+    assert np.all(np.abs(got - y64) <= 2.0 ** -7 * np.abs(y64) * 1.01 + 1e-30)
+    assert np.mean(np.abs(got - y64) / np.abs(y64)) < 2.0 ** -9      # and unbiased on average
+    # torch's bf16 rms_norm rounds once at the end; it must agree to the same bound
+    tx = torch.from_numpy(oracle.bf16_to_f32(xb)).to(torch.bfloat16)
+    tw = torch.from_numpy(oracle.bf16_to_f32(wb)).to(torch.bfloat16)
+    ty = torch.nn.functional.rms_norm(tx, (256,), tw, 1e-6).float().numpy().astype(np.float64)
+    assert np.all(np.abs(got - ty) <= 3 * 2.0 ** -8 * np.abs(y64) * 1.01 + 1e-30)

@@ -26,6 +26,10 @@ SIGNATURES = {
     "tome_fused_lmhead_logprob": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                           c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_void_p, c_size_t, c_void_p]),
+    "tome_norm_lmhead_logprob_workspace": (c_size_t, [c_int64, c_int64, c_int64]),
+    "tome_norm_lmhead_logprob": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                         c_int64, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_void_p, c_size_t, c_void_p]),
     "tome_grpo_dual_workspace": (c_size_t, [c_int64, c_int64, c_int64]),
     "tome_grpo_dual": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p,

@@ -15,9 +15,10 @@ int row_splits_for(int64_t rows, int64_t V, int vec);
 hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t rows, int64_t V,
                                    int64_t in_stride, int64_t out_stride, float temperature,
                                    const float* row_lse, hipStream_t stream);
-size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights);
-hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w1, int64_t n_tokens, int64_t H,
-                               int64_t V, int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
+size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights, bool with_norm);
+hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, float norm_eps, const void* w0,
+                               const void* w1, int64_t n_tokens, int64_t H, int64_t V, int64_t hidden_stride,
+                               int64_t weight_stride, const int32_t* targets,
                                const int32_t* row_valid, float temperature, float* out_lp, float* out_lse,
                                float* out_entropy, int32_t* out_argmax, float* out_ref_lp, float* out_k3,
                                void* workspace, hipStream_t stream);
@@ -128,7 +129,7 @@ static int check_fused(const void* hidden, const void* w, int64_t n_tokens, int6
 
 size_t tome_fused_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V) {
   if (n_tokens <= 0 || H <= 0 || V <= 0) return 0;
-  return align256(tome::fused_workspace_bytes(n_tokens, H, V, 1));
+  return align256(tome::fused_workspace_bytes(n_tokens, H, V, 1, false));
 }
 
 int tome_fused_lmhead_logprob(const void* hidden, const void* weight, int64_t n_tokens, int64_t H, int64_t V,
@@ -141,15 +142,38 @@ int tome_fused_lmhead_logprob(const void* hidden, const void* weight, int64_t n_
   if (!out_lp) return TOME_E_NULL;
   const size_t need = tome_fused_lmhead_logprob_workspace(n_tokens, H, V);
   if (!workspace || workspace_bytes < need) return TOME_E_WORKSPACE;
-  return hip_result(tome::fused_lmhead_launch(hidden, weight, nullptr, n_tokens, H, V, hidden_stride, weight_stride,
+  return hip_result(tome::fused_lmhead_launch(hidden, nullptr, 0.f, weight, nullptr, n_tokens, H, V, hidden_stride, weight_stride,
                                               targets, row_valid, temperature, out_lp, out_lse, out_entropy,
                                               out_argmax, nullptr, nullptr, workspace,
                                               static_cast<hipStream_t>(stream)));
 }
 
+size_t tome_norm_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V) {
+  if (n_tokens <= 0 || H <= 0 || V <= 0) return 0;
+  return align256(tome::fused_workspace_bytes(n_tokens, H, V, 1, true));
+}
+
+int tome_norm_lmhead_logprob(const void* hidden, const void* norm_weight, float norm_eps, const void* weight,
+                             int64_t n_tokens, int64_t H, int64_t V, int64_t hidden_stride, int64_t weight_stride,
+                             const int32_t* targets, const int32_t* row_valid, float temperature, float* out_lp,
+                             float* out_lse, float* out_entropy, int32_t* out_argmax, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+  const int rc = check_fused(hidden, weight, n_tokens, H, V, hidden_stride, weight_stride, targets, temperature);
+  if (rc != TOME_OK || n_tokens == 0) return rc;
+  if (!out_lp || !norm_weight) return TOME_E_NULL;
+  if (reinterpret_cast<uintptr_t>(norm_weight) % 16 != 0) return TOME_E_ALIGN;
+  if (!(norm_eps >= 0.f) || !isfinite(norm_eps)) return TOME_E_SHAPE;
+  const size_t need = tome_norm_lmhead_logprob_workspace(n_tokens, H, V);
+  if (!workspace || workspace_bytes < need) return TOME_E_WORKSPACE;
+  return hip_result(tome::fused_lmhead_launch(hidden, norm_weight, norm_eps, weight, nullptr, n_tokens, H, V,
+                                              hidden_stride, weight_stride, targets, row_valid, temperature, out_lp,
+                                              out_lse, out_entropy, out_argmax, nullptr, nullptr, workspace,
+                                              static_cast<hipStream_t>(stream)));
+}
+
 size_t tome_grpo_dual_workspace(int64_t n_tokens, int64_t H, int64_t V) {
   if (n_tokens <= 0 || H <= 0 || V <= 0) return 0;
-  return align256(tome::fused_workspace_bytes(n_tokens, H, V, 2));
+  return align256(tome::fused_workspace_bytes(n_tokens, H, V, 2, false));
 }
 
 int tome_grpo_dual(const void* hidden, const void* w_policy, const void* w_ref, int64_t n_tokens, int64_t H,
@@ -162,7 +186,7 @@ int tome_grpo_dual(const void* hidden, const void* w_policy, const void* w_ref, 
   if (reinterpret_cast<uintptr_t>(w_ref) % 16 != 0) return TOME_E_ALIGN;
   const size_t need = tome_grpo_dual_workspace(n_tokens, H, V);
   if (!workspace || workspace_bytes < need) return TOME_E_WORKSPACE;
-  return hip_result(tome::fused_lmhead_launch(hidden, w_policy, w_ref, n_tokens, H, V, hidden_stride, weight_stride,
+  return hip_result(tome::fused_lmhead_launch(hidden, nullptr, 0.f, w_policy, w_ref, n_tokens, H, V, hidden_stride, weight_stride,
                                               targets, row_valid, temperature, out_lp, nullptr, out_entropy,
                                               nullptr, out_ref_lp, out_k3, workspace,
                                               static_cast<hipStream_t>(stream)));

@@ -144,7 +144,8 @@ struct FusedArgs {
   const char* hidden;
   const char* weight;
   const int32_t* targets;
-  const int32_t* row_index;  // compacted valid rows, or nullptr = identity
+  const int32_t* row_index;  // compacted valid rows (position -> row of targets / outputs), or nullptr = identity
+  const int32_t* hidden_index;  // position -> row of `hidden`: row_index, or nullptr when hidden is already compact
   const int32_t* n_valid;    // device scalar, or nullptr = n_tokens
   const FusedSchedule* sched_dev;  // written by compact_rows_kernel next to n_valid, or nullptr = `sched`
   FusedPartial* partials;
@@ -294,7 +295,7 @@ __global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) 
   for (int j = 0; j < kBLoads; ++j) {
     int p = t0 + ld_row + 32 * j;
     p = p < n_valid ? p : n_valid - 1;
-    const int tok = a.row_index ? a.row_index[p] : p;
+    const int tok = a.hidden_index ? a.hidden_index[p] : p;
     boff[j] = (uint32_t)tok * a.hidden_stride_b + ld_c * 16;
   }
   uint32_t aoff[kALoads];
@@ -569,7 +570,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   for (int j = 0; j < k2Loads; ++j) {
     int p = t0 + (j * 8 + wave) * 8 + dr;
     p = p < n_valid ? p : n_valid - 1;
-    const int tok = a.row_index ? a.row_index[p] : p;
+    const int tok = a.hidden_index ? a.hidden_index[p] : p;
     pb[j] = a.hidden + (int64_t)tok * a.hidden_stride_b + dc * 16;
   }
 
@@ -776,6 +777,59 @@ __global__ __launch_bounds__(1024) void compact_rows_kernel(CompactArgs a) {
   }
 }
 
+// ---- final RMSNorm of the rows that will be multiplied ------------------------------------------
+// y = w * T(x * rsqrt(mean(x^2) + eps)) in bf16 with fp32 statistics: mx.fast.rms_norm as
+// mlx-impl/model.py:343 calls it on the last hidden states (model.py:536).  Only valid rows are
+// normalised, and they are written compactly: position p of the output is row row_index[p] of x.
+struct NormArgs {
+  const char* x;             // bf16 [n, H]
+  const uint16_t* w;         // bf16 [H]
+  char* y;                   // bf16 [n_valid, H], dense
+  const int32_t* row_index;  // or nullptr = identity
+  const int32_t* n_valid;    // or nullptr = n
+  uint32_t x_stride_b;
+  int n, H;
+  float eps;
+};
+
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(NormArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int p = blockIdx.x * 4 + (threadIdx.x >> 6);  // one wave per row
+  const int n_valid = a.n_valid ? *a.n_valid : a.n;
+  if (p >= n_valid) return;
+  const int row = a.row_index ? a.row_index[p] : p;
+  const u32x4* x = reinterpret_cast<const u32x4*>(a.x + (int64_t)row * a.x_stride_b);
+  const u32x4* w = reinterpret_cast<const u32x4*>(a.w);
+  u32x4* y = reinterpret_cast<u32x4*>(a.y + (int64_t)p * a.H * 2);
+  const int n_chunks = a.H / 8;
+  float ss = 0.f;
+  for (int c = lane; c < n_chunks; c += 64) {
+    const u32x4 v = x[c];
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float lo = bf16_lo(u[k]), hi = bf16_hi(u[k]);
+      ss = fmaf(lo, lo, ss);
+      ss = fmaf(hi, hi, ss);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+  const float inv = 1.0f / sqrtf(ss / (float)a.H + a.eps);
+  for (int c = lane; c < n_chunks; c += 64) {  // second read of the row comes from cache
+    const u32x4 v = x[c], g = w[c];
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w}, gw[4] = {g.x, g.y, g.z, g.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float lo = bf16_bits_to_f32(f32_to_bf16_bits(bf16_lo(u[k]) * inv));
+      const float hi = bf16_bits_to_f32(f32_to_bf16_bits(bf16_hi(u[k]) * inv));
+      o[k] = (uint32_t)f32_to_bf16_bits(bf16_lo(gw[k]) * lo) | ((uint32_t)f32_to_bf16_bits(bf16_hi(gw[k]) * hi) << 16);
+    }
+    y[c] = u32x4{o[0], o[1], o[2], o[3]};
+  }
+}
+
 // ---- combine -----------------------------------------------------------------------------------
 struct CombineArgs {
   const FusedPartial* partials;      // policy (or the only) weight set
@@ -789,6 +843,7 @@ struct CombineArgs {
   float* out_k3;
   int32_t* out_argmax;
   const char* hidden;  // only read when out_argmax is set
+  const int32_t* hidden_index;  // as in FusedArgs
   const char* weight;
   uint32_t hidden_stride_b;
   uint32_t weight_stride_b;
@@ -878,7 +933,7 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
     ref_lp = txr == -INFINITY ? __builtin_nanf("") : (fmaf(txr, a.scale, -mr) - fast_log2(sr.s)) * kLn2;
   }
   int amax = 0;
-  if (a.out_argmax) amax = argmax_in_block(a, tok, st.bi == 0x7fffffff ? -1 : st.bi, lane);
+  if (a.out_argmax) amax = argmax_in_block(a, a.hidden_index ? a.hidden_index[p] : p, st.bi == 0x7fffffff ? -1 : st.bi, lane);
   if (lane != 0) return;
   if (a.out_argmax) a.out_argmax[tok] = amax;
   if (a.out_lp) a.out_lp[tok] = lp;
@@ -929,15 +984,19 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   return p;
 }
 
-// Layout: [n_valid: 256 B][row_index: n_tokens int32, 256-aligned][partials per weight set].
+// Layout: [n_valid + schedule: 256 B][row_index: n_tokens int32, 256-aligned][partials per weight set]
+// [normalised hidden rows, only with a norm weight].
 static size_t off_index() { return 256; }
 static size_t off_partials(int64_t n_tokens) { return 256 + (((size_t)n_tokens * 4 + 255) & ~(size_t)255); }
+static size_t normed_bytes(int64_t n_tokens, int64_t H, bool with_norm) {
+  return with_norm ? (((size_t)n_tokens * H * 2 + 255) & ~(size_t)255) : 0;
+}
 static size_t partial_bytes(int64_t n_tokens, int64_t H, int64_t V) {
   return fused_plan(n_tokens, H, V).max_records * sizeof(FusedPartial);
 }
 
-size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights) {
-  return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, H, V);
+size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights, bool with_norm) {
+  return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, H, V) + normed_bytes(n_tokens, H, with_norm);
 }
 
 template <typename K>
@@ -959,8 +1018,9 @@ static void launch_main(const FusedArgs& a, FusedKind kind, int grid, hipStream_
   }
 }
 
-hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w1, int64_t n_tokens, int64_t H,
-                               int64_t V, int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
+hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, float norm_eps, const void* w0,
+                               const void* w1, int64_t n_tokens, int64_t H, int64_t V, int64_t hidden_stride,
+                               int64_t weight_stride, const int32_t* targets,
                                const int32_t* row_valid, float temperature, float* out_lp, float* out_lse,
                                float* out_entropy, int32_t* out_argmax, float* out_ref_lp, float* out_k3,
                                void* workspace, hipStream_t stream) {
@@ -986,10 +1046,21 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w
   a.hidden = static_cast<const char*>(hidden);
   a.targets = targets;
   a.row_index = row_index;
+  a.hidden_index = row_index;
   a.n_valid = n_valid;
   a.hidden_stride_b = (uint32_t)(hidden_stride * 2);
   a.weight_stride_b = (uint32_t)(weight_stride * 2);
   a.hidden_bytes = (uint32_t)(((n_tokens - 1) * hidden_stride + H) * 2);
+  if (norm_weight) {  // normalise the valid rows into a dense buffer and multiply that
+    char* normed = ws + off_partials(n_tokens) + (w1 ? 2 : 1) * partial_bytes(n_tokens, H, V);
+    NormArgs na{a.hidden, static_cast<const uint16_t*>(norm_weight), normed, row_index, n_valid,
+                a.hidden_stride_b, (int)n_tokens, (int)H, norm_eps};
+    hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, stream, na);
+    a.hidden = normed;
+    a.hidden_index = nullptr;
+    a.hidden_stride_b = (uint32_t)(H * 2);
+    a.hidden_bytes = (uint32_t)(n_tokens * H * 2);
+  }
   a.n_tokens = (int)n_tokens;
   a.H = (int)H;
   a.V = (int)V;
@@ -1026,6 +1097,7 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* w0, const void* w
   c.out_k3 = out_k3;
   c.out_argmax = out_argmax;
   c.hidden = a.hidden;
+  c.hidden_index = a.hidden_index;
   c.weight = static_cast<const char*>(w0);
   c.hidden_stride_b = a.hidden_stride_b;
   c.weight_stride_b = a.weight_stride_b;

@@ -208,7 +208,8 @@ def _check_fused_inputs(hidden: torch.Tensor, *weights: torch.Tensor):
 
 def fused_lmhead_logprobs(hidden: torch.Tensor, weight: torch.Tensor, targets, temperature: float = 1.0,
                           lengths=None, *, row_valid=None, want_lse: bool = False,
-                          want_entropy: bool = False, want_argmax: bool = False) -> TokenLogprobs:
+                          want_entropy: bool = False, want_argmax: bool = False,
+                          norm_weight: torch.Tensor | None = None, norm_eps: float = 1e-6) -> TokenLogprobs:
     """Log-probs of ``targets`` under softmax((hidden @ weight.T) / temperature) without the logits.
 
     ``hidden`` [..., H] bf16 (already through the final norm, mlx-impl/model.py:536),
@@ -216,6 +217,9 @@ def fused_lmhead_logprobs(hidden: torch.Tensor, weight: torch.Tensor, targets, t
     accumulated in fp32; unlike the reference the logits are not rounded to bf16.
     ``want_argmax`` adds the greedy token id (first maximum, as ``int(mx.argmax(logits))`` at
     mlx-impl/node.py:897); logits closer than fp32 accumulation noise may swap.
+    With ``norm_weight`` (bf16 [H]) ``hidden`` holds the PRE-norm states and the model's final
+    RMSNorm (``mx.fast.rms_norm(x, weight, eps)``, model.py:336-343, :536) is applied to the valid
+    rows first.
     """
     lib = _lib.load_library()
     dev, lead, h2, (w,) = _check_fused_inputs(hidden, weight)
@@ -229,12 +233,23 @@ def fused_lmhead_logprobs(hidden: torch.Tensor, weight: torch.Tensor, targets, t
         lse = torch.empty(n, dtype=torch.float32, device=dev) if want_lse else None
         ent = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
         amax = torch.empty(n, dtype=torch.int32, device=dev) if want_argmax else None
-        ws_bytes = lib.tome_fused_lmhead_logprob_workspace(n, H, V)
-        ws = _workspace(ws_bytes, dev)
-        _lib.check(lib.tome_fused_lmhead_logprob(h2.data_ptr(), w.data_ptr(), n, H, V,
-                                                 h2.stride(0) if n > 1 else H, w.stride(0),
-                                                 tg.data_ptr(), _ptr(rv), temperature, lp.data_ptr(), _ptr(lse),
-                                                 _ptr(ent), _ptr(amax), _ptr(ws), ws_bytes, _stream(dev)))
+        if norm_weight is None:
+            ws_bytes = lib.tome_fused_lmhead_logprob_workspace(n, H, V)
+            ws = _workspace(ws_bytes, dev)
+            _lib.check(lib.tome_fused_lmhead_logprob(h2.data_ptr(), w.data_ptr(), n, H, V,
+                                                     h2.stride(0) if n > 1 else H, w.stride(0),
+                                                     tg.data_ptr(), _ptr(rv), temperature, lp.data_ptr(), _ptr(lse),
+                                                     _ptr(ent), _ptr(amax), _ptr(ws), ws_bytes, _stream(dev)))
+        else:
+            if norm_weight.dtype != torch.bfloat16 or norm_weight.shape != (H,) or norm_weight.device != dev:
+                raise ValueError(f"norm_weight must be a bfloat16 [{H}] tensor on {dev}")
+            nw = norm_weight.contiguous()
+            ws_bytes = lib.tome_norm_lmhead_logprob_workspace(n, H, V)
+            ws = _workspace(ws_bytes, dev)
+            _lib.check(lib.tome_norm_lmhead_logprob(h2.data_ptr(), nw.data_ptr(), float(norm_eps), w.data_ptr(), n, H, V,
+                                                    h2.stride(0) if n > 1 else H, w.stride(0),
+                                                    tg.data_ptr(), _ptr(rv), temperature, lp.data_ptr(), _ptr(lse),
+                                                    _ptr(ent), _ptr(amax), _ptr(ws), ws_bytes, _stream(dev)))
 
     def _shaped(t):
         return None if t is None else t.reshape(lead)

@@ -54,15 +54,21 @@ class RefLogprobServicer:
     final, normalised hidden states ``(hidden [B, L, H] bf16, cache)``; only the completion rows
     are then pushed through the fused lm_head + log-softmax kernel, so logits for prompt and
     padding rows (which the reference computes at node.py:443 and discards at :449) are never
-    formed.
+    formed.  With ``final_norm_weight`` ([H] bf16) as well, ``reference_model`` returns the states
+    BEFORE the last RMSNorm (model.py:536) and that norm, too, is applied to completion rows only.
     """
 
     def __init__(self, reference_model: Callable[..., Any], device: torch.device | str = "cuda:0",
-                 max_ref_batch_size: int = 32, lm_head_weight: Optional[torch.Tensor] = None):
+                 max_ref_batch_size: int = 32, lm_head_weight: Optional[torch.Tensor] = None,
+                 final_norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 1e-6):
+        if final_norm_weight is not None and lm_head_weight is None:
+            raise ValueError("final_norm_weight needs lm_head_weight (hidden-state mode)")
         self.reference_model = reference_model
         self.device = torch.device(device)
         self.max_ref_batch_size = max_ref_batch_size     # node.py:58
         self.lm_head_weight = lm_head_weight
+        self.final_norm_weight = final_norm_weight
+        self.norm_eps = norm_eps                          # RMSNorm default, model.py:337
         self.last_ref_tokens = 0
         self.last_ref_seconds = 0.0
 
@@ -109,7 +115,8 @@ class RefLogprobServicer:
             if self.lm_head_weight is None:
                 lps = token_logprobs(out, tg, temp, row_valid=rv).lp
             else:
-                lps = fused_lmhead_logprobs(out, self.lm_head_weight, tg, temp, row_valid=rv).lp
+                lps = fused_lmhead_logprobs(out, self.lm_head_weight, tg, temp, row_valid=rv,
+                                            norm_weight=self.final_norm_weight, norm_eps=self.norm_eps).lp
             host = lps.cpu().numpy()                                      # one sync + one copy per chunk (node.py:456)
             for i, lo, n in spans:
                 p_idx, g = chunk[i][0], chunk[i][1]
