@@ -66,6 +66,27 @@ int tome_row_logprob(const void* logits, int dtype, int64_t rows, int64_t V, int
                      float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- Decode-step sampler on the same logits pass -----------------------------------
+ * Replaces, for a batch of decode rows, _sample_token(logits, temperature, top_k=20)
+ * (mlx-impl/node.py:894-907) together with the log-prob lookup
+ * float(fused_log_softmax(logits, T)[b, token]) (node.py:590,605 and 356,373) and the greedy
+ * int(mx.argmax(logits)) (node.py:602,897):
+ *   candidates   the top_k (1..32) largest logits of the row, ordered by logit descending,
+ *                equal logits by ascending token id (mx.argpartition leaves ties open)
+ *   out_token    uniforms == NULL: candidate 0 (the greedy token).  Otherwise the inverse CDF
+ *                of softmax(candidate logits / temperature) at uniforms[row] in [0, 1): the
+ *                categorical draw of node.py:906 with the randomness supplied by the caller
+ *                (MLX's own random stream cannot be reproduced).
+ *   out_lp       log-prob of out_token under the softmax over the WHOLE vocabulary
+ *   out_argmax   first maximum of the row;  out_topk_idx / out_topk_logit  [rows, top_k], the
+ *                candidates themselves (-1 / 0 past the end of a row with fewer finite logits)
+ * Masked rows give token -1.  No workspace.
+ */
+int tome_row_sample(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                    const float* uniforms, const int32_t* row_valid, float temperature, int top_k,
+                    int32_t* out_token, float* out_lp, float* out_lse, int32_t* out_argmax,
+                    int32_t* out_topk_idx, float* out_topk_logit, void* stream);
+
 /* ---- Full log-softmax matrix ------------------------------------------------------
  * fused_log_softmax(logits, temperature) as the reference returns it
  * (mlx-impl/model.py:77-89): out[r, j] = T(x[r, j] * (1/temp)) - T(lse_r), same shape

@@ -50,6 +50,13 @@ Pinning (tests/test_oracle.py):
                             as an independent library routine, brute force with
                             math.fsum.  The order of MLX's two bf16 roundings
                             (normalise, round, scale, round): parity unpinned.
+  top_k_rows / sample_top_k  np.argpartition + sort as an independent library
+                            route to the same candidate set, brute force on tiny
+                            rows, planted ties, and the law of the draw: over a
+                            fine grid of uniforms the token frequencies equal
+                            softmax(top-k logits / T) (what mx.random.categorical
+                            samples, node.py:906).  MLX's random stream itself and
+                            argpartition's order among equal logits: parity unpinned.
   process_ref_logprobs_batched  known-answer tests on a stub model
                             (alignment, empty completion, temperature 0,
                             chunking, padding id 0) and the length contract of
@@ -66,7 +73,7 @@ __all__ = [
     "bf16_round", "bf16_to_f32", "to_f64", "lse_rows", "logprob_rows", "entropy_rows",
     "argmax_rows", "k3", "lmhead_logits64", "lmhead_stats", "full_log_softmax64",
     "local_compute_logprobs_f32", "fused_log_softmax_f32", "process_ref_logprobs_batched",
-    "rms_norm64", "rms_norm_bf16",
+    "rms_norm64", "rms_norm_bf16", "top_k_rows", "sample_top_k",
 ]
 
 
@@ -178,6 +185,49 @@ def rms_norm_bf16(x: np.ndarray, weight: np.ndarray, eps: float = 1e-6) -> np.nd
     inv = (1.0 / np.sqrt(ms + float(eps))).astype(np.float32)
     t = bf16_to_f32(bf16_round(x32 * inv))
     return bf16_round(w32 * t)
+
+
+def top_k_rows(x: np.ndarray, top_k: int = 20):
+    """The ``top_k`` largest entries of each row: ``mx.argpartition(scaled_logits, size - top_k)[-top_k:]``
+    (mlx-impl/node.py:902; temperature > 0 does not change the set), returned ordered by value
+    descending, equal values by ascending index.  NaN entries are never candidates; a row with fewer
+    than ``top_k`` candidates is padded with index -1.  Returns (idx int32 [rows, top_k], val float64)."""
+    x64 = to_f64(x)
+    rows, V = x64.shape
+    idx = np.full((rows, top_k), -1, dtype=np.int32)
+    val = np.zeros((rows, top_k), dtype=np.float64)
+    for r in range(rows):
+        cand = np.flatnonzero(~np.isnan(x64[r]))
+        order = cand[np.lexsort((cand, -x64[r, cand]))][:top_k]     # value descending, then index ascending
+        idx[r, :len(order)] = order
+        val[r, :len(order)] = x64[r, order]
+    return idx, val
+
+
+def sample_top_k(x: np.ndarray, uniforms, temperature: float, top_k: int = 20):
+    """_sample_token (mlx-impl/node.py:894-907) with the randomness made explicit.
+
+    temperature == 0: ``int(mx.argmax(logits))`` (node.py:896-897).  Otherwise the categorical draw
+    over ``top_logits = (logits / temperature)[top_indices]`` (node.py:899-907) taken as the inverse
+    CDF of softmax(top_logits) at ``uniforms[r]`` in [0, 1), candidates in the order of
+    ``top_k_rows``.  Returns (token int32 [rows], lp float64 [rows]) where lp is the log-prob of the
+    token under the full softmax at ``temperature or 1.0`` (node.py:590,605)."""
+    x64 = to_f64(x)
+    rows = x64.shape[0]
+    idx, val = top_k_rows(x, top_k)
+    tok = np.empty(rows, dtype=np.int32)
+    for r in range(rows):
+        n = int((idx[r] >= 0).sum())
+        if temperature == 0 or uniforms is None:
+            tok[r] = idx[r, 0]
+            continue
+        z = val[r, :n] / float(temperature)
+        p = np.exp(z - z[0])
+        cdf = np.cumsum(p)
+        j = int(np.searchsorted(cdf, float(uniforms[r]) * cdf[-1], side="right"))
+        tok[r] = idx[r, min(j, n - 1)]
+    lp = logprob_rows(x64, tok, float(temperature) or 1.0)
+    return tok, lp
 
 
 def lmhead_stats(hidden: np.ndarray, weight: np.ndarray, targets: np.ndarray,

@@ -253,3 +253,49 @@ def test_rms_norm_bf16_is_the_closed_form_within_two_roundings():
     tw = torch.from_numpy(oracle.bf16_to_f32(wb)).to(torch.bfloat16)
     ty = torch.nn.functional.rms_norm(tx, (256,), tw, 1e-6).float().numpy().astype(np.float64)
     assert np.all(np.abs(got - ty) <= 3 * 2.0 ** -8 * np.abs(y64) * 1.01 + 1e-30)
+
+
+# ---- sampler (_sample_token, node.py:894-907) -------------------------------------------------------
+def test_top_k_rows_against_argpartition_and_bruteforce():
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((6, 500))
+    idx, val = oracle.top_k_rows(x, 20)
+    for r in range(6):
+        part = np.argpartition(x[r], x.shape[1] - 20)[-20:]          # the reference's expression, node.py:902
+        assert set(part.tolist()) == set(idx[r].tolist())
+        assert np.all(np.diff(val[r]) <= 0) and np.array_equal(val[r], x[r, idx[r]])
+    # planted ties: equal values enter by ascending index, and the cut through a tie keeps the lowest ids
+    t = np.zeros((1, 12)); t[0, [7, 2, 9]] = 5.0; t[0, [4, 1, 11, 6]] = 3.0
+    idx, _ = oracle.top_k_rows(t, 5)
+    assert idx[0].tolist() == [2, 7, 9, 1, 4]
+    # NaN is never a candidate; short rows are padded with -1
+    s = np.array([[np.nan, 1.0, -np.inf, 2.0]])
+    idx, val = oracle.top_k_rows(s, 4)
+    assert idx[0].tolist() == [3, 1, 2, -1] and val[0, 0] == 2.0
+
+
+def test_sample_top_k_law_and_limits():
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((1, 300)) * 2.0
+    T, k = 0.7, 8
+    idx, val = oracle.top_k_rows(x, k)
+    p = scipy.special.softmax(val[0] / T)                              # what a categorical over top_logits samples
+    n = 20000
+    us = (np.arange(n) + 0.5) / n
+    toks = np.array([oracle.sample_top_k(x, [u], T, k)[0][0] for u in us[::20]])   # coarse grid: 1000 draws
+    freq = np.array([(toks == i).mean() for i in idx[0]])
+    np.testing.assert_allclose(freq, p, atol=2e-3)
+    assert set(toks.tolist()) <= set(idx[0].tolist())                  # never outside the top k
+    # limits: u -> 0 is the largest logit, u -> 1 the k-th; temperature 0 is argmax with lp at T = 1
+    assert oracle.sample_top_k(x, [0.0], T, k)[0][0] == idx[0, 0] == np.argmax(x[0])
+    assert oracle.sample_top_k(x, [1.0 - 1e-12], T, k)[0][0] == idx[0, k - 1]
+    tok0, lp0 = oracle.sample_top_k(x, None, 0, k)
+    assert tok0[0] == np.argmax(x[0])
+    np.testing.assert_allclose(lp0, oracle.logprob_rows(x, tok0, 1.0))
+    # the log-prob is over the WHOLE vocabulary at the sampling temperature, not renormalised over the top k
+    tok, lp = oracle.sample_top_k(x, [0.3], T, k)
+    np.testing.assert_allclose(lp[0], scipy.special.log_softmax(x[0] / T)[tok[0]], atol=1e-12)
+    # brute force on a tiny row: k = 3 of 4 values, hand-computed CDF
+    y = np.array([[0.0, math.log(2.0), math.log(4.0), -50.0]])
+    got = [oracle.sample_top_k(y, [u], 1.0, 3)[0][0] for u in (0.0, 0.56, 0.58, 0.85, 0.86, 0.99)]
+    assert got == [2, 2, 1, 1, 0, 0]                                   # masses 4/7, 2/7, 1/7

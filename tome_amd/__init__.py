@@ -11,16 +11,18 @@ from .logprob import (  # noqa: F401
     fused_log_softmax,
     local_compute_logprobs,
     token_logprobs,
+    sample_tokens,
     fused_lmhead_logprobs,
     grpo_dual_logprobs,
     TokenLogprobs,
+    SampledTokens,
     DualLogprobs,
 )
 from .node import Prompt, Completion, PromptRollout, RefLogprobServicer  # noqa: F401
 from ._lib import TomeError, lib_path, load_library  # noqa: F401
 
 __all__ = [
-    "fused_log_softmax", "local_compute_logprobs", "token_logprobs", "fused_lmhead_logprobs",
-    "grpo_dual_logprobs", "TokenLogprobs", "DualLogprobs", "Prompt", "Completion", "PromptRollout",
+    "fused_log_softmax", "local_compute_logprobs", "token_logprobs", "sample_tokens", "fused_lmhead_logprobs",
+    "grpo_dual_logprobs", "TokenLogprobs", "SampledTokens", "DualLogprobs", "Prompt", "Completion", "PromptRollout",
     "RefLogprobServicer", "TomeError", "lib_path", "load_library",
 ]

@@ -15,6 +15,10 @@ int row_splits_for(int64_t rows, int64_t V, int vec);
 hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t rows, int64_t V,
                                    int64_t in_stride, int64_t out_stride, float temperature,
                                    const float* row_lse, hipStream_t stream);
+hipError_t row_sample_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                             const float* uniforms, const int32_t* row_valid, float temperature, int top_k,
+                             int32_t* out_token, float* out_lp, float* out_lse, int32_t* out_argmax,
+                             int32_t* out_topk_idx, float* out_topk_logit, hipStream_t stream);
 size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights, bool with_norm);
 hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, float norm_eps, const void* w0,
                                const void* w1, int64_t n_tokens, int64_t H, int64_t V, int64_t hidden_stride,
@@ -94,6 +98,21 @@ int tome_row_logprob(const void* logits, int dtype, int64_t rows, int64_t V, int
   return hip_result(tome::row_logprob_launch(logits, dtype, rows, V, row_stride, targets, row_valid, temperature,
                                              out_lp, out_lse, out_entropy, out_argmax, workspace,
                                              static_cast<hipStream_t>(stream)));
+}
+
+int tome_row_sample(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                    const float* uniforms, const int32_t* row_valid, float temperature, int top_k,
+                    int32_t* out_token, float* out_lp, float* out_lse, int32_t* out_argmax,
+                    int32_t* out_topk_idx, float* out_topk_logit, void* stream) {
+  if (dtype != TOME_F32 && dtype != TOME_BF16) return TOME_E_DTYPE;
+  if (bad_matrix(rows, V, row_stride) || top_k < 1 || top_k > 32) return TOME_E_SHAPE;
+  if (bad_temperature(temperature)) return TOME_E_TEMPERATURE;
+  if (rows == 0) return TOME_OK;
+  if (!logits || !out_token) return TOME_E_NULL;
+  if (reinterpret_cast<uintptr_t>(logits) % (dtype == TOME_F32 ? 4 : 2) != 0) return TOME_E_ALIGN;
+  return hip_result(tome::row_sample_launch(logits, dtype, rows, V, row_stride, uniforms, row_valid, temperature,
+                                            top_k, out_token, out_lp, out_lse, out_argmax, out_topk_idx,
+                                            out_topk_logit, static_cast<hipStream_t>(stream)));
 }
 
 int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows, int64_t V,

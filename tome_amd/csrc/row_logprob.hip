@@ -11,102 +11,9 @@
 // waves through LDS.  splits == 1 finishes in the same launch; otherwise per-split
 // partials go to the workspace and row_combine_kernel merges them (no float atomics, so
 // results do not depend on scheduling).
-#include "common.hpp"
+#include "row_common.hpp"
 
 namespace tome {
-
-// 256 lanes per workgroup, four 16-byte loads in flight per lane (8 workgroups = 128 KB in
-// flight per CU).  Measured on MI355X at [4096, 151936] bf16: 512/1024-lane workgroups and
-// deeper unrolling (fewer, fatter waves) are equal or slower.
-constexpr int kRowWG = 256;
-constexpr int kRowWaves = kRowWG / 64;
-constexpr int kRowUnroll = 4;
-
-template <typename T>
-struct Elem;
-template <>
-struct Elem<float> {
-  static constexpr int kVec = 4;
-  __device__ static __forceinline__ float load1(const float* p) { return *p; }
-  __device__ static __forceinline__ void unpack(const u32x4& v, float (&x)[kVec]) {
-    x[0] = __uint_as_float(v.x);
-    x[1] = __uint_as_float(v.y);
-    x[2] = __uint_as_float(v.z);
-    x[3] = __uint_as_float(v.w);
-  }
-};
-template <>
-struct Elem<uint16_t> {  // bf16 bit patterns
-  static constexpr int kVec = 8;
-  __device__ static __forceinline__ float load1(const uint16_t* p) { return bf16_bits_to_f32(*p); }
-  __device__ static __forceinline__ void unpack(const u32x4& v, float (&x)[kVec]) {
-    x[0] = bf16_lo(v.x);
-    x[1] = bf16_hi(v.x);
-    x[2] = bf16_lo(v.y);
-    x[3] = bf16_hi(v.y);
-    x[4] = bf16_lo(v.z);
-    x[5] = bf16_hi(v.z);
-    x[6] = bf16_lo(v.w);
-    x[7] = bf16_hi(v.w);
-  }
-};
-
-template <int N>
-__device__ __forceinline__ float max_of(const float (&x)[N]) {
-  float m = x[0];
-#pragma unroll
-  for (int i = 1; i + 1 < N; i += 2) m = fmaxf(m, fmaxf(x[i], x[i + 1]));  // v_max3_f32
-  if constexpr (N % 2 == 0) m = fmaxf(m, x[N - 1]);
-  return m;
-}
-
-// Fold N values of load unit `unit` into a lane's state.
-template <int N, bool ENT, bool AMAX>
-__device__ __forceinline__ void absorb(RowStat& st, const float (&x)[N], int unit, float scale) {
-  const float cm = max_of<N>(x);
-  const float mx_new = fmaxf(st.mx, cm);
-  if constexpr (AMAX) st.bi = (cm > st.mx) ? unit : st.bi;
-  const float resc = fast_exp2((st.mx - mx_new) * scale);
-  const float m = mx_new * scale;
-  float s = st.s * resc;
-  float w = ENT ? st.w * resc : 0.f;
-#pragma unroll
-  for (int i = 0; i < N; ++i) {
-    const float e = fast_exp2(fmaf(x[i], scale, -m));
-    s += e;
-    if constexpr (ENT) w = fmaf(fmaxf(x[i], kMaxFloor) * scale, e, w);
-  }
-  st.mx = mx_new;
-  st.s = s;
-  if constexpr (ENT) st.w = w;
-}
-
-// Workgroup reduction of the per-lane states; the result is valid in every lane of wave 0.
-// Fields go through LDS one by one: a whole-struct copy to LDS leaves a private stack slot behind.
-struct RowLds {
-  float mx[kRowWaves], s[kRowWaves], w[kRowWaves];
-  int bi[kRowWaves];
-};
-
-// Workgroup reduction; the result is valid in wave 0 (every lane).
-__device__ __forceinline__ RowStat block_reduce(RowStat st, float scale, RowLds& lds) {
-  constexpr int kWaves = kRowWaves;
-  stat_wave_reduce(st, scale);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (lane == 0) {
-    lds.mx[wave] = st.mx;
-    lds.s[wave] = st.s;
-    lds.w[wave] = st.w;
-    lds.bi[wave] = st.bi;
-  }
-  __syncthreads();
-  RowStat r = stat_identity();
-  if (wave == 0) {
-    if (lane < kWaves) r = RowStat{lds.mx[lane], lds.s[lane], lds.w[lane], lds.bi[lane]};
-    stat_wave_reduce(r, scale);
-  }
-  return r;
-}
 
 struct RowPartial {  // one per (row, split) in the workspace
   float mx, s, w;

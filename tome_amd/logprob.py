@@ -30,6 +30,14 @@ class TokenLogprobs(NamedTuple):
     argmax: Optional[torch.Tensor]      # int32, first maximum of the row
 
 
+class SampledTokens(NamedTuple):
+    token: torch.Tensor                 # int32, the drawn (or greedy) token id; -1 for masked rows
+    lp: torch.Tensor                    # float32, its log-prob under the full softmax
+    argmax: torch.Tensor                # int32, first maximum of the row
+    topk_idx: Optional[torch.Tensor]    # int32 [..., top_k], candidates by descending logit
+    topk_logit: Optional[torch.Tensor]  # float32 [..., top_k], their raw logits
+
+
 class DualLogprobs(NamedTuple):
     lp: torch.Tensor        # policy log-prob of the target id
     ref_lp: torch.Tensor    # reference-model log-prob of the target id
@@ -158,6 +166,52 @@ def token_logprobs(logits: torch.Tensor, targets, temperature: float = 1.0, leng
     def _shaped(t):
         return None if t is None else t.reshape(lead)
     return TokenLogprobs(_shaped(lp), _shaped(lse), _shaped(ent), _shaped(amax))
+
+
+def sample_tokens(logits: torch.Tensor, temperature: float, top_k: int = 20, *, uniforms=None,
+                  generator: Optional[torch.Generator] = None, row_valid=None, lengths=None,
+                  want_topk: bool = False) -> SampledTokens:
+    """One decode step for a batch of rows: ``_sample_token(logits, temperature, top_k)``
+    (mlx-impl/node.py:894-907) for every row at once, with the log-prob of the chosen token that
+    the decode loops look up afterwards (node.py:590,605) from the same pass.
+
+    ``temperature == 0`` is greedy (node.py:896-897) and the log-prob then uses temperature 1.0, as
+    ``temperature or 1.0`` does at node.py:590.  Otherwise the token is drawn from
+    softmax(top-k logits / temperature) by inverse CDF at ``uniforms`` (float32 in [0, 1), one per
+    row; drawn with ``torch.rand`` from ``generator`` when omitted) - candidates ordered by
+    logit descending, equal logits by ascending id.  MLX's random stream is not reproduced.
+    """
+    lib = _lib.load_library()
+    dev = _require_gpu(logits)
+    greedy = float(temperature) == 0.0
+    temperature = _check_temperature(1.0 if greedy else temperature)
+    dtype = _dtype_code(logits)
+    lead = tuple(logits.shape[:-1])
+    x = _rows_view(logits)
+    rows, V = x.shape
+    if not 1 <= int(top_k) <= 32:
+        raise ValueError("top_k must be in 1..32")
+    rv = _row_valid(lead, rows, lengths, row_valid, dev)
+    with torch.cuda.device(dev):
+        u = None
+        if not greedy:
+            if uniforms is None:
+                u = torch.rand(rows, dtype=torch.float32, device=dev, generator=generator)
+            else:
+                u = torch.as_tensor(uniforms, dtype=torch.float32, device=dev).reshape(-1).contiguous()
+                if u.numel() != rows:
+                    raise ValueError(f"uniforms must have one value per row ({rows}), got {u.numel()}")
+        tok = torch.empty(rows, dtype=torch.int32, device=dev)
+        lp = torch.empty(rows, dtype=torch.float32, device=dev)
+        amax = torch.empty(rows, dtype=torch.int32, device=dev)
+        tki = torch.empty((rows, top_k), dtype=torch.int32, device=dev) if want_topk else None
+        tkl = torch.empty((rows, top_k), dtype=torch.float32, device=dev) if want_topk else None
+        _lib.check(lib.tome_row_sample(x.data_ptr(), dtype, rows, V, x.stride(0) if rows > 1 else V, _ptr(u), _ptr(rv),
+                                       temperature, int(top_k), tok.data_ptr(), lp.data_ptr(), None, amax.data_ptr(),
+                                       _ptr(tki), _ptr(tkl), _stream(dev)))
+    return SampledTokens(tok.reshape(lead), lp.reshape(lead), amax.reshape(lead),
+                         None if tki is None else tki.reshape(*lead, top_k),
+                         None if tkl is None else tkl.reshape(*lead, top_k))
 
 
 def local_compute_logprobs(logits: torch.Tensor, ids: torch.Tensor, temp: float) -> torch.Tensor:
