@@ -146,6 +146,36 @@ def bench_fused(dev, steps, warmup):
     return {"tokens": n, "H": H, "ms": ms, "wall_ms": wall, "tflops": flop / (ms * 1e-3) / 1e12, "flop": flop}
 
 
+def bench_decode(dev, steps, warmup):
+    """One decode step's sampler + log-prob (mlx-impl/node.py:590-605) on config 1's shape: 64 rows of fp32
+    logits, top-k 20.  The buffers rotate so that the rows come from HBM, not from a warm cache."""
+    import torch
+    import tome_amd
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    rows, k, nbuf = 64, 20, 16
+    g = torch.Generator(device=dev).manual_seed(77)
+    xs = [torch.randn((rows, V), device=dev, generator=g) * 2.0 for _ in range(nbuf)]
+    u = torch.rand(rows, device=dev, generator=g)
+    tok = torch.empty(rows, dtype=torch.int32, device=dev)
+    lp = torch.empty(rows, dtype=torch.float32, device=dev)
+    ws_bytes = lib.tome_row_sample_workspace(0, rows, V, k)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    i = [0]
+
+    def step():
+        x = xs[i[0] % nbuf]
+        i[0] += 1
+        _lib.check(lib.tome_row_sample(x.data_ptr(), 0, rows, V, V, u.data_ptr(), None, 1.0, k, tok.data_ptr(),
+                                       lp.data_ptr(), None, None, None, None, ws.data_ptr(), ws_bytes, stream))
+    step()
+    torch.cuda.synchronize()
+    assert (tok >= 0).all() and (tok < V).all() and torch.isfinite(lp).all()
+    ms, wall = time_steps(step, steps, warmup)
+    return {"rows": rows, "top_k": k, "ms": ms, "bytes": rows * V * 4}
+
+
 def cpu_baseline(sample_rows=256, budget_s=12.0):
     """NumPy fp32 restatement of local_compute_logprobs (mlx-impl/node.py:400-404) on a bounded
     sample of the config-2 workload: `sample_rows` rows of bf16 logits, upcast included."""
@@ -222,6 +252,7 @@ def main():
     # the fused step is ~10x longer than a row step: half the launches keep the run short; the clocks
     # still settle (a few tens of milliseconds of back-to-back launches are needed for that)
     fused = bench_fused(dev, max(5, args.steps // 2), max(2, args.warmup // 2)) if args.only in (None, "fused") else None
+    decode = bench_decode(dev, args.steps, args.warmup) if args.only is None else None
     cpu = None if args.no_cpu else cpu_baseline()
 
     line = {
@@ -268,6 +299,17 @@ def main():
                          "roofline": f["roofline"], "dtype": "f32"})
         else:
             line["fused_lmhead"] = f
+    if decode is not None:
+        line["decode_sampler"] = {"value": decode["rows"] / (decode["ms"] * 1e-3), "unit": "sampled tokens/s",
+                                  "ms_per_step": decode["ms"], "dtype": "f32",
+                                  "config": {"workload": "one decode step: top-k sampling + log-prob + argmax, "
+                                                         "fp32 logits [64, 151936] (config 1's shape), top_k 20",
+                                             "rows": decode["rows"], "top_k": decode["top_k"], "vocab": V},
+                                  "roofline": {"bound": "hbm", "achieved": decode["bytes"] / (decode["ms"] * 1e-3) / 1e9,
+                                               "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                               "frac": decode["bytes"] / (decode["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                               "traffic": None, "kernel": "row_sample_kernel<f32> + row_sample_combine_kernel",
+                                               "bytes_per_launch": decode["bytes"]}}
     if cpu is not None:
         line["cpu_baseline"] = cpu
     print(json.dumps(line), flush=True)

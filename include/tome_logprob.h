@@ -80,12 +80,15 @@ int tome_row_logprob(const void* logits, int dtype, int64_t rows, int64_t V, int
  *   out_lp       log-prob of out_token under the softmax over the WHOLE vocabulary
  *   out_argmax   first maximum of the row;  out_topk_idx / out_topk_logit  [rows, top_k], the
  *                candidates themselves (-1 / 0 past the end of a row with fewer finite logits)
- * Masked rows give token -1.  No workspace.
+ * Masked rows give token -1.  Small batches split each row over several workgroups and need
+ * the workspace that tome_row_sample_workspace() sizes (0 for large batches).
  */
+size_t tome_row_sample_workspace(int dtype, int64_t rows, int64_t V, int top_k);
 int tome_row_sample(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
                     const float* uniforms, const int32_t* row_valid, float temperature, int top_k,
                     int32_t* out_token, float* out_lp, float* out_lse, int32_t* out_argmax,
-                    int32_t* out_topk_idx, float* out_topk_logit, void* stream);
+                    int32_t* out_topk_idx, float* out_topk_logit, void* workspace,
+                    size_t workspace_bytes, void* stream);
 
 /* ---- Full log-softmax matrix ------------------------------------------------------
  * fused_log_softmax(logits, temperature) as the reference returns it

@@ -86,10 +86,12 @@ def test_argument_checks_run_on_host():
                                                     P, None, 1.0, P, None, None, None, None, 0, None)
     assert norm(nw=None) == -1 and norm(nw=P + 4) == -6 and norm(eps=-1.0) == -3 and norm(eps=float("nan")) == -3
     assert norm(H=0) == -3 and norm() == -4
-    samp = lambda **k: lib.tome_row_sample(k.get("logits", P), k.get("dtype", 0), 4, k.get("V", 64), 64, None, None, k.get("T", 1.0),
-                                           k.get("k", 20), k.get("tok", P), None, None, None, None, None, None)
+    samp = lambda **k: lib.tome_row_sample(k.get("logits", P), k.get("dtype", 0), 4, k.get("V", 64), max(64, k.get("V", 64)), None, None, k.get("T", 1.0),
+                                           k.get("k", 20), k.get("tok", P), None, None, None, None, None, None, 0, None)
     assert samp(dtype=3) == -2 and samp(V=0) == -3 and samp(k=0) == -3 and samp(k=33) == -3 and samp(T=0.0) == -5
     assert samp(logits=None) == -1 and samp(tok=None) == -1 and samp(logits=P + 2) == -6
+    assert samp(V=151936) == -4                                      # a small batch splits its rows: workspace needed
+    assert lib.tome_row_sample_workspace(0, 4096, 151936, 20) == 0 and lib.tome_row_sample_workspace(0, 64, 151936, 20) > 0
     dual = lib.tome_grpo_dual(P, P, None, 8, 64, 100, 64, 64, P, None, 1.0, P, P, P, P, None, 0, None)
     assert dual == -1
 

@@ -20,8 +20,10 @@ SIGNATURES = {
     "tome_row_logprob_workspace": (c_size_t, [c_int64, c_int64]),
     "tome_row_logprob": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "tome_row_sample_workspace": (c_size_t, [c_int, c_int64, c_int64, c_int]),
     "tome_row_sample": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float, c_int,
-                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                c_void_p]),
     "tome_full_log_softmax": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_float,
                                       c_void_p, c_void_p, c_size_t, c_void_p]),
     "tome_fused_lmhead_logprob_workspace": (c_size_t, [c_int64, c_int64, c_int64]),

@@ -18,7 +18,8 @@ hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t
 hipError_t row_sample_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
                              const float* uniforms, const int32_t* row_valid, float temperature, int top_k,
                              int32_t* out_token, float* out_lp, float* out_lse, int32_t* out_argmax,
-                             int32_t* out_topk_idx, float* out_topk_logit, hipStream_t stream);
+                             int32_t* out_topk_idx, float* out_topk_logit, void* workspace, hipStream_t stream);
+size_t row_sample_workspace_bytes(int64_t rows, int64_t V, int dtype_vec, int top_k);
 size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights, bool with_norm);
 hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, float norm_eps, const void* w0,
                                const void* w1, int64_t n_tokens, int64_t H, int64_t V, int64_t hidden_stride,
@@ -100,19 +101,27 @@ int tome_row_logprob(const void* logits, int dtype, int64_t rows, int64_t V, int
                                              static_cast<hipStream_t>(stream)));
 }
 
+size_t tome_row_sample_workspace(int dtype, int64_t rows, int64_t V, int top_k) {
+  if (rows <= 0 || V <= 0 || top_k < 1 || top_k > 32) return 0;
+  return tome::row_sample_workspace_bytes(rows, V, dtype == TOME_F32 ? 4 : 8, top_k);
+}
+
 int tome_row_sample(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
                     const float* uniforms, const int32_t* row_valid, float temperature, int top_k,
                     int32_t* out_token, float* out_lp, float* out_lse, int32_t* out_argmax,
-                    int32_t* out_topk_idx, float* out_topk_logit, void* stream) {
+                    int32_t* out_topk_idx, float* out_topk_logit, void* workspace, size_t workspace_bytes,
+                    void* stream) {
   if (dtype != TOME_F32 && dtype != TOME_BF16) return TOME_E_DTYPE;
   if (bad_matrix(rows, V, row_stride) || top_k < 1 || top_k > 32) return TOME_E_SHAPE;
   if (bad_temperature(temperature)) return TOME_E_TEMPERATURE;
   if (rows == 0) return TOME_OK;
   if (!logits || !out_token) return TOME_E_NULL;
+  const size_t need = tome_row_sample_workspace(dtype, rows, V, top_k);
+  if (need > 0 && (!workspace || workspace_bytes < need)) return TOME_E_WORKSPACE;
   if (reinterpret_cast<uintptr_t>(logits) % (dtype == TOME_F32 ? 4 : 2) != 0) return TOME_E_ALIGN;
   return hip_result(tome::row_sample_launch(logits, dtype, rows, V, row_stride, uniforms, row_valid, temperature,
                                             top_k, out_token, out_lp, out_lse, out_argmax, out_topk_idx,
-                                            out_topk_logit, static_cast<hipStream_t>(stream)));
+                                            out_topk_logit, workspace, static_cast<hipStream_t>(stream)));
 }
 
 int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows, int64_t V,

@@ -11,20 +11,24 @@
 // kernel takes the inverse CDF of softmax(top-k logits / T), the k candidates ordered by logit
 // (descending; equal logits by ascending token id).  MLX's own random stream cannot be matched.
 //
-// One workgroup per row, two passes over the row (the second comes from L2 / MALL for decode-sized
-// batches):
+// A row is shared by `splits` workgroups (decode batches are a few dozen rows: one workgroup per row
+// would leave most of the chip idle), each making two passes over its range of the row (the second
+// comes from L2 / MALL for decode-sized batches):
 //   1. online (max, sum 2^(y-m)) for the full-vocabulary lse, and every lane's own largest element;
 //      the k-th largest of the 256 lane maxima is a lower bound `theta` of the k-th largest logit;
 //   2. every element >= theta goes to a candidate buffer in LDS (typically k + a few entries).
 // Candidates are 64-bit keys (order-preserving image of the float, then ~index), so there are no
 // ties and "the top k" is unique.  A buffer overflow (adversarial orderings only) raises theta to
 // the k-th largest of what was kept - still a lower bound - and repeats pass 2.  The final k are
-// rank-sorted by one wave.
+// rank-sorted by one wave.  With splits > 1 every workgroup leaves its k keys and its (max, sum)
+// in the workspace and row_sample_combine_kernel selects among the splits * k keys and draws.
 #include "row_common.hpp"
 
 namespace tome {
 
-constexpr int kSampCap = 2048;  // candidate keys per buffer (2 x 16 KB of LDS)
+constexpr int kSampCap = 1024;      // candidate keys per buffer in the main kernel (2 x 8 KB of LDS: 8 workgroups per CU)
+constexpr int kSampMergeCap = 2048; // in the combine kernel: up to 64 splits x 32 keys
+constexpr int kSampCached = 8;      // a lane keeps up to this many load units in registers between the passes
 constexpr int kSampMaxK = 32;  // one tightening round is then sure to drop >= 32 of the 64 sampled keys
 
 struct SampleArgs {
@@ -37,9 +41,12 @@ struct SampleArgs {
   int32_t* out_argmax;        // nullable
   int32_t* out_topk_idx;      // nullable, [rows, top_k], -1 past the end of a short row
   float* out_topk_logit;      // nullable, [rows, top_k] raw logits
+  uint64_t* part_keys;        // workspace: [rows, splits, top_k] (splits > 1)
+  float2* part_stat;          // workspace: [rows, splits] (max, sum)
   int64_t V;
   int64_t row_stride;
   int top_k;
+  int splits;
   float scale;                // log2(e) / temperature
 };
 
@@ -56,41 +63,60 @@ __device__ __forceinline__ uint64_t make_key(float x, uint32_t idx) {
 }
 __device__ __forceinline__ uint32_t key_index(uint64_t k) { return 0xFFFFFFFFu - (uint32_t)k; }
 
+template <int CAP>
 struct SampleLds {
-  uint64_t a[kSampCap];
-  uint64_t b[kSampCap];
+  uint64_t a[CAP];
+  uint64_t b[CAP];
   uint64_t top[kSampMaxK];
-  uint64_t thr;
+  uint64_t thr4[kRowWaves];
   int cnt;
   RowLds red;
 };
 
-// Number of lanes of this wave whose key is larger than this lane's (keys of lanes >= m are ignored).
+// Number of lanes of this wave whose key is larger than this lane's.  v_readlane broadcasts (the lane
+// index is uniform), not LDS-crossbar shuffles: 64 dependent ds_bpermute round trips cost microseconds.
 __device__ __forceinline__ int wave_rank(uint64_t key, int m) {
+  const uint32_t lo = (uint32_t)key, hi = (uint32_t)(key >> 32);
   int rank = 0;
+#pragma unroll 8
   for (int j = 0; j < m; ++j) {
-    const uint64_t o = __shfl(key, j, 64);
+    const uint64_t o = ((uint64_t)__builtin_amdgcn_readlane(hi, j) << 32) | (uint32_t)__builtin_amdgcn_readlane(lo, j);
     rank += o > key ? 1 : 0;
   }
   return rank;
 }
 
-// Sorted top-k of the m keys in `cur` (m <= kSampCap; 0 = empty slot) into sh.top[0..k), the rest of
+// Sorted top-k of the m keys in `cur` (m <= the buffer size; 0 = empty slot) into sh.top[0..k), the rest of
 // sh.top zeroed; returns the k-th largest key (0 if there are fewer than k).  `cur` / `other` are
 // the two LDS buffers; both are clobbered.  All lanes of the workgroup must call it.
-__device__ uint64_t select_top_k(SampleLds& sh, uint64_t* cur, uint64_t* other, int m, int k) {
+//
+// While more than 64 keys are left, a lower bound of the k-th largest is taken from a sample and the
+// keys below it are dropped:
+//   m >= 256: every wave ranks 64 keys of its own (256 distinct positions spread over the buffer);
+//             the smallest of the four ceil(k/4)-th largest has >= k sampled keys at or above it;
+//   m <  256: wave 0 ranks 64 distinct keys and takes their k-th largest.
+// Either way at least 32 sampled keys fall below the bound, so every round makes progress.
+template <class Lds>
+__device__ uint64_t select_top_k(Lds& sh, uint64_t* cur, uint64_t* other, int m, int k) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   while (m > 64) {
-    // Tighten: the k-th largest of 64 entries spread over the buffer is a lower bound of the k-th
-    // largest overall, and at least 64 - k entries fall below it.
-    if (wave == 0) {
-      const uint64_t key = cur[(int)(((int64_t)lane * m) >> 6)];
+    const bool wide = m >= kRowWG;
+    if (wide || wave == 0) {
+      const int pos = wide ? (int)(((int64_t)tid * m) >> 8) : (int)(((int64_t)lane * m) >> 6);
+      const uint64_t key = cur[pos];
       const int rank = wave_rank(key, 64);
-      if (rank == k - 1) sh.thr = key;  // equal keys (empty slots only) write the same value
-      if (lane == 0) sh.cnt = 0;
+      const int want = wide ? (k + kRowWaves - 1) / kRowWaves : k;
+      if (lane == 0) sh.thr4[wave] = 0;  // stays 0 (no bound) when fewer than `want` sampled keys are real
+      __builtin_amdgcn_wave_barrier();
+      if (key != 0 && rank == want - 1) sh.thr4[wave] = key;
     }
+    if (tid == 0) sh.cnt = 0;
     __syncthreads();
-    const uint64_t thr = sh.thr;
+    uint64_t thr = sh.thr4[0];
+    if (wide) {
+#pragma unroll
+      for (int w = 1; w < kRowWaves; ++w) thr = sh.thr4[w] < thr ? sh.thr4[w] : thr;
+    }
     for (int i = tid; i < m; i += kRowWG) {
       const uint64_t key = cur[i];
       if (key >= thr && key != 0) other[atomicAdd(&sh.cnt, 1)] = key;
@@ -107,8 +133,8 @@ __device__ uint64_t select_top_k(SampleLds& sh, uint64_t* cur, uint64_t* other, 
   if (m > 64) m = 64;  // unreachable, see above
   if (wave == 0) {
     const uint64_t key = lane < m ? cur[lane] : 0;
-    const int rank = wave_rank(key, 64);
-    sh.top[lane] = 0;
+    const int rank = wave_rank(key, m);  // lanes >= m hold 0 and outrank nobody
+    sh.top[lane & (kSampMaxK - 1)] = 0;
     __builtin_amdgcn_wave_barrier();
     if (key != 0 && rank < k) sh.top[rank] = key;
   }
@@ -116,146 +142,38 @@ __device__ uint64_t select_top_k(SampleLds& sh, uint64_t* cur, uint64_t* other, 
   return sh.top[k - 1];
 }
 
-template <typename T, bool VECTOR>
-__global__ __launch_bounds__(kRowWG) void row_sample_kernel(SampleArgs a) {
-  constexpr int kVec = VECTOR ? Elem<T>::kVec : 1;
-  __shared__ SampleLds sh;
-  const int64_t r = blockIdx.x;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+// Lower bound of the k-th largest element of this workgroup's range from the lanes' own maxima (-inf
+// for a lane that saw nothing): each wave extracts its ceil(k/4) largest lane maxima one by one (a
+// wave-wide max, then the first lane that holds it steps aside), and the smallest of the four results
+// has at least k lane maxima at or above it.  Values only - any element with that value passes.
+template <class Lds>
+__device__ uint64_t bound_from_lane_maxima(Lds& sh, float lane_max, int k) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int want = (k + kRowWaves - 1) / kRowWaves;
+  float v = lane_max, kth = -INFINITY;
+  for (int t = 0; t < want; ++t) {
+    float m = v;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    kth = m;
+    const uint64_t holders = __ballot(v == m);
+    if (holders == 0) break;  // cannot happen (lane maxima are never NaN); guards the ctz below
+    if (lane == __builtin_ctzll(holders)) v = -INFINITY;
+  }
+  if (lane == 0) sh.thr4[wave] = (uint64_t)float_key(kth) << 32;
+  __syncthreads();
+  uint64_t thr = sh.thr4[0];
+#pragma unroll
+  for (int w = 1; w < kRowWaves; ++w) thr = sh.thr4[w] < thr ? sh.thr4[w] : thr;
+  __syncthreads();
+  return thr;
+}
+
+// Wave 0: draw among the sorted candidates in sh.top and write the row's outputs.  `tot` holds the
+// full-vocabulary (max, sum) in every lane.
+template <class Lds>
+__device__ __forceinline__ void finish_sample(const SampleArgs& a, Lds& sh, int64_t r, const RowStat& tot, int lane) {
   const int k = a.top_k;
-
-  if (a.row_valid && a.row_valid[r] == 0) {  // masked row: not read
-    if (tid == 0) {
-      a.out_token[r] = -1;
-      if (a.out_lp) a.out_lp[r] = 0.f;
-      if (a.out_lse) a.out_lse[r] = 0.f;
-      if (a.out_argmax) a.out_argmax[r] = -1;
-    }
-    if (tid < k) {
-      if (a.out_topk_idx) a.out_topk_idx[r * k + tid] = -1;
-      if (a.out_topk_logit) a.out_topk_logit[r * k + tid] = 0.f;
-    }
-    return;
-  }
-
-  const T* row = static_cast<const T*>(a.logits) + r * a.row_stride;
-  const int64_t n_units = a.V / kVec;
-  const int n_tail = (int)(a.V - n_units * kVec);  // single elements after the last whole unit (lane 0)
-
-  // ---- pass 1: full-vocabulary statistics and this lane's own maximum --------------------------
-  RowStat st = stat_identity();
-  if constexpr (VECTOR) {
-    const u32x4* p = reinterpret_cast<const u32x4*>(row);
-    int64_t u = tid;
-    for (; u + (kRowUnroll - 1) * kRowWG < n_units; u += kRowUnroll * kRowWG) {
-      u32x4 v[kRowUnroll];
-#pragma unroll
-      for (int q = 0; q < kRowUnroll; ++q) v[q] = p[u + q * kRowWG];
-#pragma unroll
-      for (int q = 0; q < kRowUnroll; ++q) {
-        float x[kVec];
-        Elem<T>::unpack(v[q], x);
-        absorb<kVec, false, true>(st, x, (int)(u + q * kRowWG), a.scale);
-      }
-    }
-    for (; u < n_units; u += kRowWG) {
-      float x[kVec];
-      Elem<T>::unpack(p[u], x);
-      absorb<kVec, false, true>(st, x, (int)u, a.scale);
-    }
-    if (tid == 0) {
-      for (int e = 0; e < n_tail; ++e) {
-        float x[1] = {Elem<T>::load1(row + n_units * kVec + e)};
-        absorb<1, false, true>(st, x, (int)(n_units + e), a.scale);
-      }
-    }
-  } else {
-    for (int64_t u = tid; u < n_units; u += kRowWG) {
-      float x[1] = {Elem<T>::load1(row + u)};
-      absorb<1, false, true>(st, x, (int)u, a.scale);
-    }
-  }
-  // This lane's maximum as a key: the first element of unit st.bi that equals st.mx.
-  uint64_t lane_key = 0;
-  if (st.bi != 0x7fffffff) {
-    const int64_t first = st.bi < n_units ? (int64_t)st.bi * kVec : n_units * kVec + (st.bi - n_units);
-    const int count = st.bi < n_units ? kVec : 1;
-    int64_t idx = first;
-    for (int i = count - 1; i >= 0; --i)
-      if (Elem<T>::load1(row + first + i) == st.mx) idx = first + i;
-    lane_key = make_key(st.mx, (uint32_t)idx);
-  }
-  const RowStat tot = block_reduce(st, a.scale, sh.red);  // valid in wave 0
-
-  // ---- theta: k-th largest lane maximum (rows that fit the buffer skip the bound) ----------------
-  uint64_t theta = 0;
-  if (a.V > kSampCap) {
-    sh.a[tid] = lane_key;
-    __syncthreads();
-    theta = select_top_k(sh, sh.a, sh.b, kRowWG, k);
-    __syncthreads();
-  }
-
-  // ---- pass 2: collect every element >= theta ---------------------------------------------------
-  int m = 0;
-  for (;;) {
-    if (tid == 0) sh.cnt = 0;
-    __syncthreads();
-    const float theta_val = theta == 0 ? -INFINITY : key_float((uint32_t)(theta >> 32));
-    auto offer = [&](float x, int64_t idx) {
-      if (x >= theta_val) {
-        const uint64_t key = make_key(x, (uint32_t)idx);
-        if (key >= theta) {
-          const int pos = atomicAdd(&sh.cnt, 1);
-          if (pos < kSampCap) sh.a[pos] = key;
-        }
-      }
-    };
-    if constexpr (VECTOR) {
-      const u32x4* p = reinterpret_cast<const u32x4*>(row);
-      int64_t u = tid;
-      for (; u + (kRowUnroll - 1) * kRowWG < n_units; u += kRowUnroll * kRowWG) {
-        u32x4 v[kRowUnroll];
-#pragma unroll
-        for (int q = 0; q < kRowUnroll; ++q) v[q] = p[u + q * kRowWG];
-#pragma unroll
-        for (int q = 0; q < kRowUnroll; ++q) {
-          float x[kVec];
-          Elem<T>::unpack(v[q], x);
-          if (max_of<kVec>(x) >= theta_val) {
-#pragma unroll
-            for (int i = 0; i < kVec; ++i) offer(x[i], (u + q * kRowWG) * kVec + i);
-          }
-        }
-      }
-      for (; u < n_units; u += kRowWG) {
-        float x[kVec];
-        Elem<T>::unpack(p[u], x);
-        if (max_of<kVec>(x) >= theta_val) {
-#pragma unroll
-          for (int i = 0; i < kVec; ++i) offer(x[i], u * kVec + i);
-        }
-      }
-      if (tid == 0)
-        for (int e = 0; e < n_tail; ++e) offer(Elem<T>::load1(row + n_units * kVec + e), n_units * kVec + e);
-    } else {
-      for (int64_t u = tid; u < n_units; u += kRowWG) offer(Elem<T>::load1(row + u), u);
-    }
-    __syncthreads();
-    const int offered = sh.cnt;
-    __syncthreads();
-    if (offered <= kSampCap) {
-      m = offered;
-      break;
-    }
-    // Overflow: the k-th largest of the kSampCap keys that were kept is a strictly higher lower bound.
-    theta = select_top_k(sh, sh.a, sh.b, kSampCap, k);
-    __syncthreads();
-  }
-
-  // ---- final selection, draw and outputs (wave 0) -----------------------------------------------
-  select_top_k(sh, sh.a, sh.b, m, k);
-  if (wave != 0) return;
   const uint64_t key = lane < k ? sh.top[lane] : 0;
   const bool have = key != 0;
   const float x = have ? key_float((uint32_t)(key >> 32)) : -INFINITY;
@@ -292,23 +210,263 @@ __global__ __launch_bounds__(kRowWG) void row_sample_kernel(SampleArgs a) {
   if (a.out_lse) a.out_lse[r] = (m2 + log2s) * kLn2;
 }
 
+// CACHED: the host promises that a lane owns at most kSampCached load units (short ranges: decode
+// batches split over many workgroups); they are loaded once and both passes run from registers.
+template <typename T, bool VECTOR, bool CACHED>
+__global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) void row_sample_kernel(SampleArgs a) {
+  static_assert(VECTOR || !CACHED, "the cached variant is for 16-byte units");
+  constexpr int kVec = VECTOR ? Elem<T>::kVec : 1;
+  __shared__ SampleLds<kSampCap> sh;
+  const int64_t r = blockIdx.x / a.splits;
+  const int split = blockIdx.x % a.splits;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int k = a.top_k;
+
+  if (a.row_valid && a.row_valid[r] == 0) {  // masked row: not read
+    if (split != 0) return;
+    if (tid == 0) {
+      a.out_token[r] = -1;
+      if (a.out_lp) a.out_lp[r] = 0.f;
+      if (a.out_lse) a.out_lse[r] = 0.f;
+      if (a.out_argmax) a.out_argmax[r] = -1;
+    }
+    if (tid < k) {
+      if (a.out_topk_idx) a.out_topk_idx[r * k + tid] = -1;
+      if (a.out_topk_logit) a.out_topk_logit[r * k + tid] = 0.f;
+    }
+    return;
+  }
+
+  const T* row = static_cast<const T*>(a.logits) + r * a.row_stride;
+  const int64_t n_units = a.V / kVec;
+  const int64_t per_split = (n_units + a.splits - 1) / a.splits;
+  const int64_t u0 = per_split * split;
+  const int64_t u1 = (u0 + per_split < n_units) ? u0 + per_split : n_units;
+  // single elements after the last whole unit: lane 0 of the last split
+  const int n_tail = split == a.splits - 1 ? (int)(a.V - n_units * kVec) : 0;
+
+  // ---- pass 1: full-vocabulary statistics and this lane's own maximum --------------------------
+  RowStat st = stat_identity();
+  u32x4 cached[CACHED ? kSampCached : 1];
+  if constexpr (CACHED) {
+    const u32x4* p = reinterpret_cast<const u32x4*>(row);
+#pragma unroll
+    for (int q = 0; q < kSampCached; ++q) {  // unconditional (clamped) loads: all eight in flight together
+      const int64_t u = u0 + tid + q * kRowWG;
+      cached[q] = p[u < u1 ? u : 0];         // unit 0 exists (checked on the host)
+    }
+#pragma unroll
+    for (int q = 0; q < kSampCached; ++q)
+      if (u0 + tid + q * kRowWG < u1) {
+        float x[kVec];
+        Elem<T>::unpack(cached[q], x);
+        absorb<kVec, false, true>(st, x, (int)(u0 + tid + q * kRowWG), a.scale);
+        __builtin_amdgcn_sched_barrier(0);  // one unit at a time: hoisting all eight overflows the registers
+      }
+    if (tid == 0) {
+      for (int e = 0; e < n_tail; ++e) {
+        float x[1] = {Elem<T>::load1(row + n_units * kVec + e)};
+        absorb<1, false, true>(st, x, (int)(n_units + e), a.scale);
+      }
+    }
+  } else if constexpr (VECTOR) {
+    const u32x4* p = reinterpret_cast<const u32x4*>(row);
+    int64_t u = u0 + tid;
+    for (; u + (kRowUnroll - 1) * kRowWG < u1; u += kRowUnroll * kRowWG) {
+      u32x4 v[kRowUnroll];
+#pragma unroll
+      for (int q = 0; q < kRowUnroll; ++q) v[q] = p[u + q * kRowWG];
+#pragma unroll
+      for (int q = 0; q < kRowUnroll; ++q) {
+        float x[kVec];
+        Elem<T>::unpack(v[q], x);
+        absorb<kVec, false, true>(st, x, (int)(u + q * kRowWG), a.scale);
+      }
+    }
+    for (; u < u1; u += kRowWG) {
+      float x[kVec];
+      Elem<T>::unpack(p[u], x);
+      absorb<kVec, false, true>(st, x, (int)u, a.scale);
+    }
+    if (tid == 0) {
+      for (int e = 0; e < n_tail; ++e) {
+        float x[1] = {Elem<T>::load1(row + n_units * kVec + e)};
+        absorb<1, false, true>(st, x, (int)(n_units + e), a.scale);
+      }
+    }
+  } else {
+    for (int64_t u = u0 + tid; u < u1; u += kRowWG) {
+      float x[1] = {Elem<T>::load1(row + u)};
+      absorb<1, false, true>(st, x, (int)u, a.scale);
+    }
+  }
+  // This lane's maximum as a key: the first element of unit st.bi that equals st.mx.
+  uint64_t lane_key = 0;
+  if (st.bi != 0x7fffffff) {
+    const int64_t first = st.bi < n_units ? (int64_t)st.bi * kVec : n_units * kVec + (st.bi - n_units);
+    const int count = st.bi < n_units ? kVec : 1;
+    int64_t idx = first;
+    for (int i = count - 1; i >= 0; --i)
+      if (Elem<T>::load1(row + first + i) == st.mx) idx = first + i;
+    lane_key = make_key(st.mx, (uint32_t)idx);
+  }
+  const RowStat tot = block_reduce(st, a.scale, sh.red);  // valid in wave 0
+
+  // ---- theta: k-th largest lane maximum (ranges that fit the buffer skip the bound) --------------
+  uint64_t theta = 0;
+  if ((u1 - u0) * kVec + n_tail > kSampCap) {
+    theta = bound_from_lane_maxima(sh, lane_key != 0 ? st.mx : -INFINITY, k);
+  }
+
+  // ---- pass 2: collect every element >= theta ---------------------------------------------------
+  int m = 0;
+  for (;;) {
+    if (tid == 0) sh.cnt = 0;
+    __syncthreads();
+    const float theta_val = theta == 0 ? -INFINITY : key_float((uint32_t)(theta >> 32));
+    auto offer = [&](float x, int64_t idx) {
+      if (x >= theta_val) {
+        const uint64_t key = make_key(x, (uint32_t)idx);
+        if (key >= theta) {
+          const int pos = atomicAdd(&sh.cnt, 1);
+          if (pos < kSampCap) sh.a[pos] = key;
+        }
+      }
+    };
+    if constexpr (CACHED) {
+      // Opaque to the optimiser, so that the keys and element indices below are formed where they are
+      // used (rarely) instead of being hoisted out of the retry loop into a hundred live registers.
+      uint32_t first_elem = (uint32_t)((u0 + tid) * kVec);
+      asm volatile("" : "+v"(first_elem));
+#pragma unroll
+      for (int q = 0; q < kSampCached; ++q)
+        asm volatile("" : "+v"(cached[q].x), "+v"(cached[q].y), "+v"(cached[q].z), "+v"(cached[q].w));
+#pragma unroll
+      for (int q = 0; q < kSampCached; ++q)
+        if (u0 + tid + q * kRowWG < u1) {
+          float x[kVec];
+          Elem<T>::unpack(cached[q], x);
+          if (max_of<kVec>(x) >= theta_val) {
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) offer(x[i], first_elem + (uint32_t)(q * kRowWG * kVec + i));
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      if (tid == 0)
+        for (int e = 0; e < n_tail; ++e) offer(Elem<T>::load1(row + n_units * kVec + e), n_units * kVec + e);
+    } else if constexpr (VECTOR) {
+      const u32x4* p = reinterpret_cast<const u32x4*>(row);
+      int64_t u = u0 + tid;
+      for (; u + (kRowUnroll - 1) * kRowWG < u1; u += kRowUnroll * kRowWG) {
+        u32x4 v[kRowUnroll];
+#pragma unroll
+        for (int q = 0; q < kRowUnroll; ++q) v[q] = p[u + q * kRowWG];
+#pragma unroll
+        for (int q = 0; q < kRowUnroll; ++q) {
+          float x[kVec];
+          Elem<T>::unpack(v[q], x);
+          if (max_of<kVec>(x) >= theta_val) {
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) offer(x[i], (u + q * kRowWG) * kVec + i);
+          }
+        }
+      }
+      for (; u < u1; u += kRowWG) {
+        float x[kVec];
+        Elem<T>::unpack(p[u], x);
+        if (max_of<kVec>(x) >= theta_val) {
+#pragma unroll
+          for (int i = 0; i < kVec; ++i) offer(x[i], u * kVec + i);
+        }
+      }
+      if (tid == 0)
+        for (int e = 0; e < n_tail; ++e) offer(Elem<T>::load1(row + n_units * kVec + e), n_units * kVec + e);
+    } else {
+      for (int64_t u = u0 + tid; u < u1; u += kRowWG) offer(Elem<T>::load1(row + u), u);
+    }
+    __syncthreads();
+    const int offered = sh.cnt;
+    __syncthreads();
+    if (offered <= kSampCap) {
+      m = offered;
+      break;
+    }
+    // Overflow: the k-th largest of the kSampCap keys that were kept is a strictly higher lower bound.
+    theta = select_top_k(sh, sh.a, sh.b, kSampCap, k);
+    __syncthreads();
+  }
+
+  // ---- final selection ---------------------------------------------------------------------------
+  select_top_k(sh, sh.a, sh.b, m, k);
+  if (wave != 0) return;
+  if (a.splits == 1) {
+    finish_sample(a, sh, r, tot, lane);
+  } else {
+    const int64_t slot = r * a.splits + split;
+    if (lane < k) a.part_keys[slot * k + lane] = sh.top[lane];
+    if (lane == 0) a.part_stat[slot] = float2{tot.mx, tot.s};
+  }
+}
+
+// splits > 1: one workgroup per row merges the splits' candidates and statistics and draws.
+__global__ __launch_bounds__(kRowWG) void row_sample_combine_kernel(SampleArgs a) {
+  __shared__ SampleLds<kSampMergeCap> sh;
+  const int64_t r = blockIdx.x;
+  if (a.row_valid && a.row_valid[r] == 0) return;  // outputs already written by the main kernel
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int k = a.top_k, m = a.splits * k;         // <= 64 * 32 = kSampMergeCap
+  for (int i = tid; i < m; i += kRowWG) sh.a[i] = a.part_keys[r * m + i];
+  __syncthreads();
+  select_top_k(sh, sh.a, sh.b, m, k);
+  if (wave != 0) return;
+  RowStat st = stat_identity();
+  if (lane < a.splits) {
+    const float2 p = a.part_stat[r * a.splits + lane];
+    st.mx = p.x;
+    st.s = p.y;
+  }
+  stat_wave_reduce(st, a.scale);
+  finish_sample(a, sh, r, st, lane);
+}
+
+int row_splits_for(int64_t rows, int64_t V, int vec);
+
+static size_t align256s(size_t b) { return (b + 255) & ~(size_t)255; }
+size_t row_sample_workspace_bytes(int64_t rows, int64_t V, int dtype_vec, int top_k) {
+  const int splits = row_splits_for(rows, V, dtype_vec);
+  if (splits == 1) return 0;
+  return align256s((size_t)rows * splits * top_k * sizeof(uint64_t)) + align256s((size_t)rows * splits * sizeof(float2));
+}
+
 hipError_t row_sample_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
                              const float* uniforms, const int32_t* row_valid, float temperature, int top_k,
                              int32_t* out_token, float* out_lp, float* out_lse, int32_t* out_argmax,
-                             int32_t* out_topk_idx, float* out_topk_logit, hipStream_t stream) {
+                             int32_t* out_topk_idx, float* out_topk_logit, void* workspace, hipStream_t stream) {
   const int esize = dtype == 0 ? 4 : 2;
   const int vec = 16 / esize;
   const bool vector_ok = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && (row_stride % vec == 0);
+  // The workspace is sized for the vector layout; the element-wise instantiation uses the same split count.
+  const int splits = row_splits_for(rows, V, vec);
+  char* ws = static_cast<char*>(workspace);
   SampleArgs a{logits, uniforms, row_valid, out_token, out_lp, out_lse, out_argmax, out_topk_idx, out_topk_logit,
-               V, row_stride, top_k, kLog2e / temperature};
-  const dim3 grid((unsigned)rows), block(kRowWG);
+               reinterpret_cast<uint64_t*>(ws),
+               reinterpret_cast<float2*>(ws + align256s((size_t)rows * splits * top_k * sizeof(uint64_t))),
+               V, row_stride, top_k, splits, kLog2e / temperature};
+  const dim3 grid((unsigned)(rows * splits)), block(kRowWG);
+  const int64_t units_per_split = (V / vec + splits - 1) / splits;
+  const bool cached = vector_ok && V >= vec && units_per_split <= (int64_t)kSampCached * kRowWG;
   if (dtype == 0) {
-    if (vector_ok) hipLaunchKernelGGL((row_sample_kernel<float, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((row_sample_kernel<float, false>), grid, block, 0, stream, a);
+    if (cached) hipLaunchKernelGGL((row_sample_kernel<float, true, true>), grid, block, 0, stream, a);
+    else if (vector_ok) hipLaunchKernelGGL((row_sample_kernel<float, true, false>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((row_sample_kernel<float, false, false>), grid, block, 0, stream, a);
   } else {
-    if (vector_ok) hipLaunchKernelGGL((row_sample_kernel<uint16_t, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((row_sample_kernel<uint16_t, false>), grid, block, 0, stream, a);
+    if (cached) hipLaunchKernelGGL((row_sample_kernel<uint16_t, true, true>), grid, block, 0, stream, a);
+    else if (vector_ok) hipLaunchKernelGGL((row_sample_kernel<uint16_t, true, false>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((row_sample_kernel<uint16_t, false, false>), grid, block, 0, stream, a);
   }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || splits == 1) return e;
+  hipLaunchKernelGGL(row_sample_combine_kernel, dim3((unsigned)rows), block, 0, stream, a);
   return hipGetLastError();
 }
 

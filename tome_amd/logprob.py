@@ -206,9 +206,11 @@ def sample_tokens(logits: torch.Tensor, temperature: float, top_k: int = 20, *, 
         amax = torch.empty(rows, dtype=torch.int32, device=dev)
         tki = torch.empty((rows, top_k), dtype=torch.int32, device=dev) if want_topk else None
         tkl = torch.empty((rows, top_k), dtype=torch.float32, device=dev) if want_topk else None
+        ws_bytes = lib.tome_row_sample_workspace(dtype, rows, V, int(top_k))
+        ws = _workspace(ws_bytes, dev)
         _lib.check(lib.tome_row_sample(x.data_ptr(), dtype, rows, V, x.stride(0) if rows > 1 else V, _ptr(u), _ptr(rv),
                                        temperature, int(top_k), tok.data_ptr(), lp.data_ptr(), None, amax.data_ptr(),
-                                       _ptr(tki), _ptr(tkl), _stream(dev)))
+                                       _ptr(tki), _ptr(tkl), _ptr(ws), ws_bytes, _stream(dev)))
     return SampledTokens(tok.reshape(lead), lp.reshape(lead), amax.reshape(lead),
                          None if tki is None else tki.reshape(*lead, top_k),
                          None if tkl is None else tkl.reshape(*lead, top_k))
