@@ -19,10 +19,14 @@ from .logprob import (  # noqa: F401
     DualLogprobs,
 )
 from .node import Prompt, Completion, PromptRollout, RefLogprobServicer  # noqa: F401
+from .wire import (  # noqa: F401
+    PackedRefChunk, pack_ref_work, scatter_ref_logprobs, rollout_response_to_json, rollout_response_from_json,
+)
 from ._lib import TomeError, lib_path, load_library  # noqa: F401
 
 __all__ = [
     "fused_log_softmax", "local_compute_logprobs", "token_logprobs", "sample_tokens", "fused_lmhead_logprobs",
     "grpo_dual_logprobs", "TokenLogprobs", "SampledTokens", "DualLogprobs", "Prompt", "Completion", "PromptRollout",
-    "RefLogprobServicer", "TomeError", "lib_path", "load_library",
+    "RefLogprobServicer", "PackedRefChunk", "pack_ref_work", "scatter_ref_logprobs",
+    "rollout_response_to_json", "rollout_response_from_json", "TomeError", "lib_path", "load_library",
 ]

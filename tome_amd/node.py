@@ -17,6 +17,7 @@ from typing import Any, Callable, List, Optional, Sequence
 import numpy as np
 import torch
 
+from .wire import pack_ref_work, scatter_ref_logprobs
 from .logprob import fused_lmhead_logprobs, token_logprobs
 
 logger = logging.getLogger(__name__)
@@ -81,47 +82,25 @@ class RefLogprobServicer:
                                      temperature: float = 1.0) -> None:
         """Synchronous body of ``_process_ref_logprobs_batched`` (the reference's coroutine has no awaits)."""
         t0 = time.perf_counter()
-        all_work = []                                                     # node.py:409-414
-        for p_idx, p in enumerate(prompts):
-            p_toks = list(p.tokens)
-            for g in range(G):
-                all_work.append((p_idx, g, p_toks, list(results[p_idx].completions[g].tokens)))
-
         num_toks = 0
         temp = temperature or 1.0                                         # node.py:451
-        for c0 in range(0, len(all_work), self.max_ref_batch_size):      # node.py:419-421
-            chunk = all_work[c0:c0 + self.max_ref_batch_size]
-            seqs = [p + c[:-1] if c else p for _, _, p, c in chunk]      # node.py:427-437
-            max_len = max(len(s) for s in seqs)
-            ids = np.zeros((len(chunk), max_len), dtype=np.int64)        # right-pad with id 0, node.py:440
-            targets = np.zeros((len(chunk), max_len), dtype=np.int32)
-            valid = np.zeros((len(chunk), max_len), dtype=np.int32)
-            spans = []
-            for i, (s, (_, _, p_toks, c_toks)) in enumerate(zip(seqs, chunk)):
-                ids[i, :len(s)] = s
-                if c_toks:                                               # rows p_len-1 .. p_len-2+len(c), node.py:449
-                    lo = len(p_toks) - 1
-                    if lo < 0:
-                        raise ValueError("a prompt needs at least one token to score its completion")
-                    targets[i, lo:lo + len(c_toks)] = c_toks
-                    valid[i, lo:lo + len(c_toks)] = 1
-                    spans.append((i, lo, len(c_toks)))
-            if not spans:
+        # work list, chunks of max_ref_batch_size, right-padding with id 0: node.py:409-441
+        for chunk in pack_ref_work(prompts, results, G, self.max_ref_batch_size):
+            if chunk.n_scored == 0:                                      # only empty completions (node.py:428-432)
                 continue
-            full_ids = torch.from_numpy(ids).to(self.device)
+            full_ids = torch.from_numpy(chunk.ids).to(self.device)
             out, _ = self.reference_model(full_ids, cache=None)           # node.py:443
-            tg = torch.from_numpy(targets).to(self.device)
-            rv = torch.from_numpy(valid).to(self.device)
+            tg = torch.from_numpy(chunk.targets).to(self.device)
+            rv = torch.from_numpy(chunk.valid).to(self.device)
             if self.lm_head_weight is None:
                 lps = token_logprobs(out, tg, temp, row_valid=rv).lp
             else:
                 lps = fused_lmhead_logprobs(out, self.lm_head_weight, tg, temp, row_valid=rv,
                                             norm_weight=self.final_norm_weight, norm_eps=self.norm_eps).lp
-            host = lps.cpu().numpy()                                      # one sync + one copy per chunk (node.py:456)
-            for i, lo, n in spans:
-                p_idx, g = chunk[i][0], chunk[i][1]
-                results[p_idx].completions[g].ref_log_probs.extend(host[i, lo:lo + n].tolist())  # node.py:458
-                num_toks += n
+            # one sync + one copy per chunk (node.py:456), of the scored positions only: rows
+            # p_len-1 .. p_len-2+len(c) of each sequence (node.py:449), packed in row-major order
+            flat = lps[rv.bool()].cpu().numpy()
+            num_toks += scatter_ref_logprobs(chunk, flat, results)        # node.py:457-458
 
         elapsed = time.perf_counter() - t0
         self.last_ref_tokens, self.last_ref_seconds = num_toks, elapsed
