@@ -6,7 +6,7 @@ resident in HBM.  The headline workload is BASELINE config 2 (the Qwen3-0.6B GRP
 ref-logprob shape: bf16 logits [8 x 512, 151936] with a padding mask); the same JSON line
 also carries the unmasked variant and the fused lm_head + log-softmax kernel at config 3.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only row|fused]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only row|fused|decode]
 
 Prints ONE JSON line on stdout.  Everything else goes to stderr.
 """
@@ -220,7 +220,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["row", "fused"], default=None)
+    ap.add_argument("--only", choices=["row", "fused", "decode"], default=None)
     ap.add_argument("--row-variant", choices=["both", "mask", "all"], default="both",
                     help="time config 2 with its padding mask, without it, or both (profiling runs pick one)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -252,7 +252,7 @@ def main():
     # the fused step is ~10x longer than a row step: half the launches keep the run short; the clocks
     # still settle (a few tens of milliseconds of back-to-back launches are needed for that)
     fused = bench_fused(dev, max(5, args.steps // 2), max(2, args.warmup // 2)) if args.only in (None, "fused") else None
-    decode = bench_decode(dev, args.steps, args.warmup) if args.only is None else None
+    decode = bench_decode(dev, args.steps, args.warmup) if args.only in (None, "decode") else None
     cpu = None if args.no_cpu else cpu_baseline()
 
     line = {
@@ -300,16 +300,21 @@ def main():
         else:
             line["fused_lmhead"] = f
     if decode is not None:
-        line["decode_sampler"] = {"value": decode["rows"] / (decode["ms"] * 1e-3), "unit": "sampled tokens/s",
-                                  "ms_per_step": decode["ms"], "dtype": "f32",
-                                  "config": {"workload": "one decode step: top-k sampling + log-prob + argmax, "
-                                                         "fp32 logits [64, 151936] (config 1's shape), top_k 20",
-                                             "rows": decode["rows"], "top_k": decode["top_k"], "vocab": V},
-                                  "roofline": {"bound": "hbm", "achieved": decode["bytes"] / (decode["ms"] * 1e-3) / 1e9,
-                                               "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                               "frac": decode["bytes"] / (decode["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                                               "traffic": None, "kernel": "row_sample_kernel<f32> + row_sample_combine_kernel",
-                                               "bytes_per_launch": decode["bytes"]}}
+        gbs = decode["bytes"] / (decode["ms"] * 1e-3) / 1e9
+        d = {"value": decode["rows"] / (decode["ms"] * 1e-3), "unit": "sampled tokens/s",
+             "ms_per_step": decode["ms"], "dtype": "f32",
+             "config": {"workload": "one decode step: top-k sampling + log-prob + argmax, "
+                                    "fp32 logits [64, 151936] (config 1's shape), top_k 20",
+                        "rows": decode["rows"], "top_k": decode["top_k"], "vocab": V},
+             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                          "kernel": "row_sample_kernel<f32> + row_sample_combine_kernel",
+                          "bytes_per_launch": decode["bytes"]}}
+        if row is None and fused is None:
+            line.update({"value": d["value"], "unit": d["unit"], "ms_per_step": d["ms_per_step"], "config": d["config"],
+                         "roofline": d["roofline"]})
+        else:
+            line["decode_sampler"] = d
     if cpu is not None:
         line["cpu_baseline"] = cpu
     print(json.dumps(line), flush=True)

@@ -140,3 +140,28 @@ def test_sampler_strided_and_unaligned_rows(dev):
     np.testing.assert_array_equal(got.topk_idx.cpu().numpy(), want_idx)
     np.testing.assert_array_equal(got.token.cpu().numpy(), want_tok)
     np.testing.assert_allclose(got.lp.cpu().numpy(), want_lp, atol=1e-4, rtol=0)
+
+
+def test_decode_step_graph_replays_match_eager(dev):
+    """The sampler captured as a HIP graph: several replays on changing inputs, with eager work and
+    synchronisations between them, each compared with the eager call on the same inputs."""
+    rng = np.random.default_rng(12)
+    rows, V = 48, 30011
+    logits = torch.zeros((rows, V), dtype=torch.float32, device=dev)
+    step = tome_amd.DecodeStepGraph(logits, 0.8, 20)
+    for it in range(4):
+        x = torch.from_numpy((rng.standard_normal((rows, V)) * (1.0 + it)).astype(np.float32)).to(dev)
+        u = torch.from_numpy(rng.random(rows).astype(np.float32)).to(dev)
+        step.logits.copy_(x)
+        step.uniforms.copy_(u)
+        got = step.replay()
+        torch.cuda.synchronize()
+        tok, lp, amax = got.token.clone(), got.lp.clone(), got.argmax.clone()
+        want = tome_amd.sample_tokens(x, 0.8, 20, uniforms=u)                 # eager, on the same inputs
+        torch.cuda.synchronize()
+        assert torch.equal(tok, want.token) and torch.equal(amax, want.argmax)
+        assert torch.equal(lp, want.lp)                                        # same kernels, same order: bit-identical
+        # unrelated eager work between replays
+        (x @ x[:8].T).sum().item()
+    x64 = x.cpu().numpy().astype(np.float64)
+    np.testing.assert_array_equal(amax.cpu().numpy(), np.argmax(x64, -1))

@@ -12,6 +12,7 @@ from .logprob import (  # noqa: F401
     local_compute_logprobs,
     token_logprobs,
     sample_tokens,
+    DecodeStepGraph,
     fused_lmhead_logprobs,
     grpo_dual_logprobs,
     TokenLogprobs,
@@ -25,7 +26,7 @@ from .wire import (  # noqa: F401
 from ._lib import TomeError, lib_path, load_library  # noqa: F401
 
 __all__ = [
-    "fused_log_softmax", "local_compute_logprobs", "token_logprobs", "sample_tokens", "fused_lmhead_logprobs",
+    "fused_log_softmax", "local_compute_logprobs", "token_logprobs", "sample_tokens", "DecodeStepGraph", "fused_lmhead_logprobs",
     "grpo_dual_logprobs", "TokenLogprobs", "SampledTokens", "DualLogprobs", "Prompt", "Completion", "PromptRollout",
     "RefLogprobServicer", "PackedRefChunk", "pack_ref_work", "scatter_ref_logprobs",
     "rollout_response_to_json", "rollout_response_from_json", "TomeError", "lib_path", "load_library",

@@ -216,6 +216,38 @@ def sample_tokens(logits: torch.Tensor, temperature: float, top_k: int = 20, *, 
                          None if tkl is None else tkl.reshape(*lead, top_k))
 
 
+class DecodeStepGraph:
+    """``sample_tokens`` for one fixed decode-batch shape, captured once as a HIP graph and replayed.
+
+    A decode loop (mlx-impl/node.py:575-612) calls the sampler once per generated token with the
+    same shapes; replaying a captured graph removes the per-call host work (argument checks, output
+    allocation, two kernel launches).  ``logits`` and ``uniforms`` are the static input buffers: write
+    the step's logits and fresh uniforms into them (``copy_``, ``uniform_``), call ``replay()``, read
+    ``token`` / ``lp`` / ``argmax``.  The kernels allocate nothing and clear nothing with memsets,
+    so every replay computes exactly what the eager call does.
+    """
+
+    def __init__(self, logits: torch.Tensor, temperature: float, top_k: int = 20, *, uniforms: Optional[torch.Tensor] = None):
+        dev = _require_gpu(logits)
+        self.logits = logits
+        rows = logits.numel() // logits.shape[-1]
+        self.uniforms = uniforms if uniforms is not None else torch.rand(rows, dtype=torch.float32, device=dev)
+        self.temperature, self.top_k = float(temperature), int(top_k)
+        self._stream = torch.cuda.Stream(device=dev)       # default priority
+        self._graph = torch.cuda.CUDAGraph()
+        self._stream.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(self._stream):
+            sample_tokens(self.logits, self.temperature, self.top_k, uniforms=self.uniforms)   # warm-up outside capture
+        self._stream.synchronize()
+        with torch.cuda.graph(self._graph, stream=self._stream):
+            out = sample_tokens(self.logits, self.temperature, self.top_k, uniforms=self.uniforms)
+        self.token, self.lp, self.argmax = out.token, out.lp, out.argmax
+
+    def replay(self) -> SampledTokens:
+        self._graph.replay()
+        return SampledTokens(self.token, self.lp, self.argmax, None, None)
+
+
 def local_compute_logprobs(logits: torch.Tensor, ids: torch.Tensor, temp: float) -> torch.Tensor:
     """Drop-in for the closure at mlx-impl/node.py:400-404.
 
