@@ -90,36 +90,29 @@ __device__ __forceinline__ int wave_rank(uint64_t key, int m) {
 // sh.top zeroed; returns the k-th largest key (0 if there are fewer than k).  `cur` / `other` are
 // the two LDS buffers; both are clobbered.  All lanes of the workgroup must call it.
 //
-// While more than 64 keys are left, a lower bound of the k-th largest is taken from a sample and the
-// keys below it are dropped:
-//   m >= 256: every wave ranks 64 keys of its own (256 distinct positions spread over the buffer);
-//             the smallest of the four ceil(k/4)-th largest has >= k sampled keys at or above it;
-//   m <  256: wave 0 ranks 64 distinct keys and takes their k-th largest.
-// Either way at least 32 sampled keys fall below the bound, so every round makes progress.
+// Up to 256 keys are ranked directly: lane i counts the keys larger than key i (uniform LDS
+// addresses: broadcast reads).  More than that are first thinned by a lower bound of the k-th
+// largest from a sample: every wave ranks 64 keys of its own (256 distinct positions spread over the
+// buffer), and the smallest of the four ceil(k/4)-th largest has >= k sampled keys at or above it;
+// at least 32 sampled keys fall below it, so every round makes progress.
 template <class Lds>
 __device__ uint64_t select_top_k(Lds& sh, uint64_t* cur, uint64_t* other, int m, int k) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  while (m > 64) {
-    const bool wide = m >= kRowWG;
-    if (wide || wave == 0) {
-      const int pos = wide ? (int)(((int64_t)tid * m) >> 8) : (int)(((int64_t)lane * m) >> 6);
-      const uint64_t key = cur[pos];
-      const int rank = wave_rank(key, 64);
-      const int want = wide ? (k + kRowWaves - 1) / kRowWaves : k;
-      if (lane == 0) sh.thr4[wave] = 0;  // stays 0 (no bound) when fewer than `want` sampled keys are real
-      __builtin_amdgcn_wave_barrier();
-      if (key != 0 && rank == want - 1) sh.thr4[wave] = key;
-    }
+  while (m > kRowWG) {
+    const uint64_t key = cur[(int)(((int64_t)tid * m) >> 8)];
+    const int rank = wave_rank(key, 64);
+    const int want = (k + kRowWaves - 1) / kRowWaves;
+    if (lane == 0) sh.thr4[wave] = 0;  // stays 0 (no bound) when fewer than `want` sampled keys are real
+    __builtin_amdgcn_wave_barrier();
+    if (key != 0 && rank == want - 1) sh.thr4[wave] = key;
     if (tid == 0) sh.cnt = 0;
     __syncthreads();
     uint64_t thr = sh.thr4[0];
-    if (wide) {
 #pragma unroll
-      for (int w = 1; w < kRowWaves; ++w) thr = sh.thr4[w] < thr ? sh.thr4[w] : thr;
-    }
+    for (int w = 1; w < kRowWaves; ++w) thr = sh.thr4[w] < thr ? sh.thr4[w] : thr;
     for (int i = tid; i < m; i += kRowWG) {
-      const uint64_t key = cur[i];
-      if (key >= thr && key != 0) other[atomicAdd(&sh.cnt, 1)] = key;
+      const uint64_t key2 = cur[i];
+      if (key2 >= thr && key2 != 0) other[atomicAdd(&sh.cnt, 1)] = key2;
     }
     __syncthreads();
     const int kept = sh.cnt;
@@ -130,14 +123,13 @@ __device__ uint64_t select_top_k(Lds& sh, uint64_t* cur, uint64_t* other, int m,
     cur = other;
     other = t;
   }
-  if (m > 64) m = 64;  // unreachable, see above
-  if (wave == 0) {
-    const uint64_t key = lane < m ? cur[lane] : 0;
-    const int rank = wave_rank(key, m);  // lanes >= m hold 0 and outrank nobody
-    sh.top[lane & (kSampMaxK - 1)] = 0;
-    __builtin_amdgcn_wave_barrier();
-    if (key != 0 && rank < k) sh.top[rank] = key;
-  }
+  if (m > kRowWG) m = kRowWG;  // unreachable, see above
+  const uint64_t key = tid < m ? cur[tid] : 0;
+  int rank = 0;
+  for (int j = 0; j < m; ++j) rank += cur[j] > key ? 1 : 0;
+  if (tid < kSampMaxK) sh.top[tid] = 0;
+  __syncthreads();
+  if (key != 0 && rank < k) sh.top[rank] = key;
   __syncthreads();
   return sh.top[k - 1];
 }
@@ -152,9 +144,13 @@ __device__ uint64_t bound_from_lane_maxima(Lds& sh, float lane_max, int k) {
   const int want = (k + kRowWaves - 1) / kRowWaves;
   float v = lane_max, kth = -INFINITY;
   for (int t = 0; t < want; ++t) {
-    float m = v;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    float m = v;  // wave-wide maximum: four DPP steps inside the rows, two exchanges across them
+    m = fmaxf(m, wave_exchange<0>(m));
+    m = fmaxf(m, wave_exchange<1>(m));
+    m = fmaxf(m, wave_exchange<2>(m));
+    m = fmaxf(m, wave_exchange<3>(m));
+    m = fmaxf(m, wave_exchange<4>(m));
+    m = fmaxf(m, wave_exchange<5>(m));
     kth = m;
     const uint64_t holders = __ballot(v == m);
     if (holders == 0) break;  // cannot happen (lane maxima are never NaN); guards the ctz below
@@ -303,13 +299,28 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
   // This lane's maximum as a key: the first element of unit st.bi that equals st.mx.
   uint64_t lane_key = 0;
   if (st.bi != 0x7fffffff) {
-    const int64_t first = st.bi < n_units ? (int64_t)st.bi * kVec : n_units * kVec + (st.bi - n_units);
-    const int count = st.bi < n_units ? kVec : 1;
-    int64_t idx = first;
-    for (int i = count - 1; i >= 0; --i)
-      if (Elem<T>::load1(row + first + i) == st.mx) idx = first + i;
+    int64_t idx = -1;
+    if constexpr (CACHED) {  // the unit is still in registers
+#pragma unroll
+      for (int q = kSampCached - 1; q >= 0; --q)
+        if (st.bi == (int)(u0 + tid + q * kRowWG)) {
+          float x[kVec];
+          Elem<T>::unpack(cached[q], x);
+#pragma unroll
+          for (int i = kVec - 1; i >= 0; --i)
+            if (x[i] == st.mx) idx = (int64_t)st.bi * kVec + i;
+        }
+    }
+    if (idx < 0) {  // a tail element, or the streaming variants: read the unit again
+      const int64_t first = st.bi < n_units ? (int64_t)st.bi * kVec : n_units * kVec + (st.bi - n_units);
+      const int count = st.bi < n_units ? kVec : 1;
+      idx = first;
+      for (int i = count - 1; i >= 0; --i)
+        if (Elem<T>::load1(row + first + i) == st.mx) idx = first + i;
+    }
     lane_key = make_key(st.mx, (uint32_t)idx);
   }
+  if (tid == 0) sh.cnt = 0;
   const RowStat tot = block_reduce(st, a.scale, sh.red);  // valid in wave 0
 
   // ---- theta: k-th largest lane maximum (ranges that fit the buffer skip the bound) --------------
@@ -319,10 +330,9 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
   }
 
   // ---- pass 2: collect every element >= theta ---------------------------------------------------
+  // sh.cnt is zero here: cleared before the reduction's barrier above, and again after an overflow.
   int m = 0;
   for (;;) {
-    if (tid == 0) sh.cnt = 0;
-    __syncthreads();
     const float theta_val = theta == 0 ? -INFINITY : key_float((uint32_t)(theta >> 32));
     auto offer = [&](float x, int64_t idx) {
       if (x >= theta_val) {
@@ -386,13 +396,14 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
     }
     __syncthreads();
     const int offered = sh.cnt;
-    __syncthreads();
     if (offered <= kSampCap) {
       m = offered;
       break;
     }
     // Overflow: the k-th largest of the kSampCap keys that were kept is a strictly higher lower bound.
+    __syncthreads();
     theta = select_top_k(sh, sh.a, sh.b, kSampCap, k);
+    if (tid == 0) sh.cnt = 0;
     __syncthreads();
   }
 
