@@ -94,7 +94,29 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 def _stream(dev: torch.device) -> int:
+    """Raw hipStream_t of torch's current stream on ``dev`` (the launch stream of every call)."""
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)   # a fraction of the cost of the Stream object
+    if raw is not None and dev.index is not None:
+        return raw(dev.index)
     return torch.cuda.current_stream(dev).cuda_stream
+
+
+class _on_device:
+    """``torch.cuda.device(dev)`` that does nothing when ``dev`` is already current (the usual case):
+    the HIP launches of the library go to the current device, so it has to be the tensors' one."""
+
+    def __init__(self, dev: torch.device):
+        idx = dev.index if dev.index is not None else torch.cuda.current_device()
+        self._guard = None if idx == torch.cuda.current_device() else torch.cuda.device(idx)
+
+    def __enter__(self):
+        if self._guard is not None:
+            self._guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self._guard is not None:
+            return self._guard.__exit__(*exc)
+        return False
 
 
 def _as_i32(t, n: int, dev: torch.device, what: str) -> torch.Tensor:
@@ -152,7 +174,7 @@ def token_logprobs(logits: torch.Tensor, targets, temperature: float = 1.0, leng
     rows, V = x.shape
     tg = _as_i32(targets, rows, dev, "targets")
     rv = _row_valid(lead, rows, lengths, row_valid, dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         lp = torch.empty(rows, dtype=torch.float32, device=dev)
         lse = torch.empty(rows, dtype=torch.float32, device=dev) if want_lse else None
         ent = torch.empty(rows, dtype=torch.float32, device=dev) if want_entropy else None
@@ -192,7 +214,7 @@ def sample_tokens(logits: torch.Tensor, temperature: float, top_k: int = 20, *, 
     if not 1 <= int(top_k) <= 32:
         raise ValueError("top_k must be in 1..32")
     rv = _row_valid(lead, rows, lengths, row_valid, dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         u = None
         if not greedy:
             if uniforms is None:
@@ -266,7 +288,7 @@ def fused_log_softmax(logits: torch.Tensor, temperature: float = 1.0) -> torch.T
     dtype = _dtype_code(logits)
     x = _rows_view(logits)
     rows, V = x.shape
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         out = torch.empty((rows, V), dtype=logits.dtype, device=dev)
         row_lse = torch.empty(rows, dtype=torch.float32, device=dev)
         ws_bytes = lib.tome_row_logprob_workspace(rows, V)
@@ -316,7 +338,7 @@ def fused_lmhead_logprobs(hidden: torch.Tensor, weight: torch.Tensor, targets, t
     V = w.shape[0]
     tg = _as_i32(targets, n, dev, "targets")
     rv = _row_valid(lead, n, lengths, row_valid, dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         lp = torch.empty(n, dtype=torch.float32, device=dev)
         lse = torch.empty(n, dtype=torch.float32, device=dev) if want_lse else None
         ent = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
@@ -362,7 +384,7 @@ def grpo_dual_logprobs(hidden: torch.Tensor, w_policy: torch.Tensor, w_ref: torc
     V = wp.shape[0]
     tg = _as_i32(targets, n, dev, "targets")
     rv = _row_valid(lead, n, lengths, row_valid, dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         outs = [torch.empty(n, dtype=torch.float32, device=dev) for _ in range(4)]
         ws_bytes = lib.tome_grpo_dual_workspace(n, H, V)
         ws = _workspace(ws_bytes, dev)
