@@ -57,6 +57,11 @@ Pinning (tests/test_oracle.py):
                             softmax(top-k logits / T) (what mx.random.categorical
                             samples, node.py:906).  MLX's random stream itself and
                             argpartition's order among equal logits: parity unpinned.
+  rollout_decode / judge_decode  known-answer tests on a scripted transition-table
+                            model at temperature 0 (hand-derived token lists): EOS
+                            kept with its log-prob in Rollout and dropped in Judge,
+                            the first token never checked in Rollout, the
+                            max_tokens cut, eos / 0 fed to finished rows.
   process_ref_logprobs_batched  known-answer tests on a stub model
                             (alignment, empty completion, temperature 0,
                             chunking, padding id 0) and the length contract of
@@ -73,7 +78,7 @@ __all__ = [
     "bf16_round", "bf16_to_f32", "to_f64", "lse_rows", "logprob_rows", "entropy_rows",
     "argmax_rows", "k3", "lmhead_logits64", "lmhead_stats", "full_log_softmax64",
     "local_compute_logprobs_f32", "fused_log_softmax_f32", "process_ref_logprobs_batched",
-    "rms_norm64", "rms_norm_bf16", "top_k_rows", "sample_top_k",
+    "rms_norm64", "rms_norm_bf16", "top_k_rows", "sample_top_k", "rollout_decode", "judge_decode",
 ]
 
 
@@ -331,6 +336,79 @@ def process_ref_logprobs_batched(prompts: Sequence, results: Sequence, G: int,
             results[p_idx].completions[g].ref_log_probs.extend(lps.tolist())  # node.py:458
             num_toks += len(c_toks)
     return num_toks
+
+
+def _draw(logits_row: np.ndarray, u, temperature: float, top_k: int):
+    """One call of _sample_token or argmax (node.py:598-602) and the log-prob lookup (node.py:605)."""
+    tok, lp = sample_top_k(logits_row[None, :], None if u is None else [u], temperature, top_k)
+    return int(tok[0]), float(lp[0])
+
+
+def rollout_decode(model_step: Callable[[np.ndarray], np.ndarray], last_logits: np.ndarray, G: int,
+                   temperature: float, max_tokens: int, eos_token_id: int, uniforms, top_k: int = 20) -> list:
+    """The sampling half of _rollout_batched, mlx-impl/node.py:556-612, row by row as the reference does.
+
+    ``uniforms[step][row]`` replaces MLX's random stream (step 0 = first tokens).
+    ``model_step(tokens int64 [N]) -> logits [N, V]`` stands for the model call of node.py:585."""
+    num_prompts = last_logits.shape[0]
+    active_tokens, active_lps = [], []
+    for p_idx in range(num_prompts):                                       # node.py:556-571
+        for g_idx in range(G):
+            u = None if temperature == 0 else uniforms[0][p_idx * G + g_idx]
+            token, lp = _draw(to_f64(last_logits[p_idx]), u, temperature, top_k)
+            active_tokens.append(token)
+            active_lps.append(lp)
+    total = num_prompts * G
+    seq = [{"tokens": [active_tokens[i]], "log_probs": [active_lps[i]]} for i in range(total)]   # node.py:574
+    finished = [False] * total                                             # node.py:575
+    for step in range(max_tokens - 1):                                     # node.py:578
+        if all(finished):
+            break
+        logits = to_f64(model_step(np.array(active_tokens, dtype=np.int64)))   # node.py:583-585
+        new_active = []
+        for b in range(total):                                             # node.py:592-610
+            if finished[b]:
+                new_active.append(eos_token_id)
+                continue
+            u = None if temperature == 0 else uniforms[step + 1][b]
+            token, lp = _draw(logits[b], u, temperature, top_k)
+            seq[b]["tokens"].append(token)
+            seq[b]["log_probs"].append(lp)
+            if token == eos_token_id or len(seq[b]["tokens"]) >= max_tokens:
+                finished[b] = True
+            new_active.append(token)
+        active_tokens = new_active
+    return seq
+
+
+def judge_decode(model_step: Callable[[np.ndarray], np.ndarray], first_logits: np.ndarray, temperature: float,
+                 max_tokens: int, eos_token_id: int, uniforms, top_k: int = 20) -> list:
+    """The sampling half of a Judge chunk, mlx-impl/node.py:325-374."""
+    B = first_logits.shape[0]
+    active_tokens, results = [], []
+    for i in range(B):                                                     # node.py:334-342
+        u = None if temperature == 0 else uniforms[0][i]
+        token, lp = _draw(to_f64(first_logits[i]), u, temperature, top_k)
+        active_tokens.append(token)
+        results.append({"tokens": [token], "log_probs": [lp]})
+    active = [True] * B                                                    # node.py:344
+    for step in range(max_tokens - 1):                                     # node.py:346
+        if not any(active):
+            break
+        inputs = np.array([t if active[i] else 0 for i, t in enumerate(active_tokens)], dtype=np.int64)  # :350
+        logits = to_f64(model_step(inputs))
+        for i in range(B):                                                 # node.py:357-374
+            if not active[i]:
+                continue
+            u = None if temperature == 0 else uniforms[step + 1][i]
+            token, lp = _draw(logits[i], u, temperature, top_k)
+            active_tokens[i] = token
+            if token == eos_token_id:
+                active[i] = False
+            else:
+                results[i]["tokens"].append(token)
+                results[i]["log_probs"].append(lp)
+    return results
 
 
 def _brute_logprob(row: Sequence[float], target: int, temperature: float = 1.0) -> float:

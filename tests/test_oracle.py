@@ -299,3 +299,61 @@ def test_sample_top_k_law_and_limits():
     y = np.array([[0.0, math.log(2.0), math.log(4.0), -50.0]])
     got = [oracle.sample_top_k(y, [u], 1.0, 3)[0][0] for u in (0.0, 0.56, 0.58, 0.85, 0.86, 0.99)]
     assert got == [2, 2, 1, 1, 0, 0]                                   # masses 4/7, 2/7, 1/7
+
+
+# ---- decode loops (node.py:556-612 Rollout, node.py:325-374 Judge) ----------------------------------
+def _table_model(table):
+    """Greedy transition table: logits[b] peak at table[token]."""
+    V = len(table)
+    def step(tokens):
+        out = np.full((len(tokens), V), -5.0)
+        out[np.arange(len(tokens)), [table[int(t)] for t in tokens]] = 5.0
+        return out
+    return step
+
+
+def test_decode_loops_known_answers_at_temperature_zero():
+    EOS = 0
+    table = [0, 2, 3, 0, 5, 6, 7, 1, 8]                 # 1 -> 2 -> 3 -> 0 (EOS);  4 -> 5 -> 6 -> 7 -> 1 -> ...
+    model = _table_model(table)
+    first = np.full((2, 9), -5.0); first[0, 1] = 5.0; first[1, 4] = 5.0          # prompt 0 starts at 1, prompt 1 at 4
+    lp_peak = 5.0 - np.log(np.exp(5.0) + 8 * np.exp(-5.0))
+    # Rollout, G = 2, max_tokens = 5: EOS is kept with its log-prob; the other chain is cut at 5 tokens
+    seq = oracle.rollout_decode(model, first, 2, 0.0, 5, EOS, None)
+    assert [s["tokens"] for s in seq] == [[1, 2, 3, 0], [1, 2, 3, 0], [4, 5, 6, 7, 1], [4, 5, 6, 7, 1]]
+    for s in seq:
+        assert len(s["log_probs"]) == len(s["tokens"])                            # tests/test_grpo.py:78-80
+        np.testing.assert_allclose(s["log_probs"], lp_peak, atol=1e-12)
+    # Judge, same model: EOS ends the item and is NOT recorded
+    res = oracle.judge_decode(model, first, 0.0, 5, EOS, None)
+    assert [r["tokens"] for r in res] == [[1, 2, 3], [4, 5, 6, 7, 1]]
+    # a first token equal to EOS: Rollout does not check it and goes on feeding it; Judge keeps it too (node.py:334-342)
+    first_eos = np.full((1, 9), -5.0); first_eos[0, EOS] = 5.0
+    assert oracle.rollout_decode(model, first_eos, 1, 0.0, 3, EOS, None)[0]["tokens"] == [0, 0]      # table[0] = 0 = EOS -> finished
+    assert oracle.judge_decode(model, first_eos, 0.0, 3, EOS, None)[0]["tokens"] == [0]
+    # finished rows are fed eos (Rollout) / 0 (Judge): record the inputs the model sees
+    seen = []
+    def spy(tokens):
+        seen.append([int(t) for t in tokens]); return model(tokens)
+    oracle.rollout_decode(spy, first, 1, 0.0, 6, 7, None)                          # EOS id 7 here
+    assert seen[3] == [0, 7] and seen[4] == [0, 7]                                 # chain 1 drew 7 at step 3 and is fed 7 afterwards
+    seen.clear()
+    oracle.judge_decode(spy, first, 0.0, 6, 3, None)                               # EOS id 3: item 0 stops after [1, 2]
+    assert seen[2][0] == 0                                                         # inactive item is fed 0 (node.py:350)
+
+
+def test_decode_loops_use_the_sampler_with_temperature():
+    rng = np.random.default_rng(31)
+    V = 40
+    W = rng.standard_normal((V, V)) * 2.0
+    model = lambda tokens: W[np.asarray(tokens)]
+    first = rng.standard_normal((2, V)) * 2.0
+    us = rng.random((6, 4))
+    seq = oracle.rollout_decode(model, first, 2, 0.8, 6, -1, us, top_k=5)
+    assert all(len(s["tokens"]) == 6 for s in seq)
+    # every token is one of the 5 best of its row, and its log-prob is the full-vocabulary one at T = 0.8
+    for b, s in enumerate(seq):
+        rows = [first[b // 2]] + [W[t] for t in s["tokens"][:-1]]
+        for row, tok, lp in zip(rows, s["tokens"], s["log_probs"]):
+            assert tok in np.argsort(-row)[:5]
+            np.testing.assert_allclose(lp, scipy.special.log_softmax(row / 0.8)[tok], atol=1e-12)
