@@ -392,7 +392,7 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 // Fold one wave tile (NBV x NBT blocks of 16x16) into the per-token running states.  Element e of
 // block i holds vocab row  vw0 + i*16 + 4*g + e  (g = lane / 16) for the token of block column j.
-template <bool ENT, int NBV, int NBT>
+template <bool ENT, bool AMAX, int NBV, int NBT>
 __device__ __forceinline__ void fold_tile16(f32x4v (&acc)[NBV][NBT], RowStat (&st)[NBT], float (&tx)[NBT],
                                             const int (&tgt)[NBT], int vw0, int g, bool partial_tile, int V,
                                             float scale) {
@@ -424,8 +424,10 @@ __device__ __forceinline__ void fold_tile16(f32x4v (&acc)[NBV][NBT], RowStat (&s
 #pragma unroll
     for (int i = 0; i < NBV; ++i) {
       const float bm = raw_max3(acc[i][j][0], acc[i][j][1], raw_max(acc[i][j][2], acc[i][j][3]));
-      const bool up = bm > cm;
-      bi = up ? (vw0 + i * 16) : bi;  // first row of the 16-row block
+      if constexpr (AMAX) {  // two more VALU operations per block: only when the argmax is asked for
+        const bool up = bm > cm;
+        bi = up ? (vw0 + i * 16) : bi;  // first row of the 16-row block
+      }
       cm = raw_max(cm, bm);
     }
     const float resc = fast_exp2((st[j].mx - cm) * scale);
@@ -533,7 +535,7 @@ __device__ __forceinline__ void pair_reads() {
   }
 }
 
-template <bool ENT>
+template <bool ENT, bool AMAX>
 __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -710,7 +712,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   for (int vt = vt0; vt < vt1; ++vt) {
     for (int kt = 0; kt < nk; ++kt) do_step();
     const int v0 = vt * k2BV;
-    fold_tile16<ENT>(acc, st, tx, tgt, v0 + wave_v * kWaveV, g, v0 + k2BV > a.V, a.V, a.scale);
+    fold_tile16<ENT, AMAX>(acc, st, tx, tgt, v0 + wave_v * kWaveV, g, v0 + k2BV > a.V, a.V, a.scale);
 #pragma unroll
     for (int i = 0; i < k2NBV; ++i)
 #pragma unroll
@@ -1004,15 +1006,21 @@ static void allow_big_lds(K kernel, int bytes) {
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
-template <bool ENT>
-static void launch_main(const FusedArgs& a, FusedKind kind, int grid, hipStream_t stream) {
+template <bool ENT, bool AMAX>
+static void launch_dma(const FusedArgs& a, int grid, hipStream_t stream) {
   static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
   if (!attr_set) {
-    allow_big_lds(&fused_lmhead_dma_kernel<ENT>, k2LdsTotal);
+    allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX>, k2LdsTotal);
     attr_set = true;
   }
+  hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX>), dim3((unsigned)grid), dim3(k2WG), k2LdsTotal, stream, a);
+}
+
+template <bool ENT>
+static void launch_main(const FusedArgs& a, FusedKind kind, int grid, bool want_argmax, hipStream_t stream) {
   if (kind == kDma) {
-    hipLaunchKernelGGL(fused_lmhead_dma_kernel<ENT>, dim3((unsigned)grid), dim3(k2WG), k2LdsTotal, stream, a);
+    if (want_argmax) launch_dma<ENT, true>(a, grid, stream);
+    else launch_dma<ENT, false>(a, grid, stream);
   } else {
     hipLaunchKernelGGL(fused_lmhead_kernel<ENT>, dim3((unsigned)grid), dim3(kFusedWG), 0, stream, a);
   }
@@ -1075,12 +1083,12 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, floa
 
   a.weight = static_cast<const char*>(w0);
   a.partials = p0;
-  if (out_entropy) launch_main<true>(a, plan.kind, plan.grid, stream);
-  else launch_main<false>(a, plan.kind, plan.grid, stream);
+  if (out_entropy) launch_main<true>(a, plan.kind, plan.grid, out_argmax != nullptr, stream);
+  else launch_main<false>(a, plan.kind, plan.grid, out_argmax != nullptr, stream);
   if (w1) {
     a.weight = static_cast<const char*>(w1);
     a.partials = p1;
-    launch_main<false>(a, plan.kind, plan.grid, stream);
+    launch_main<false>(a, plan.kind, plan.grid, false, stream);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
