@@ -662,27 +662,31 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 
   // 16 MFMAs on four vocab blocks; the group barriers then put one LDS read or DMA request behind
   // every MFMA (or every second one), so that its issue hides under the MFMA's execution.
-  auto mfma_half = [&](int i0, bf16x8 (&fa)[4], bf16x8 (&fb)[k2NBT]) {
+  // `fresh`: the first K sub-step of a vocab tile starts from a zero C operand, which saves clearing
+  // the 128 accumulator registers after every fold.
+  auto mfma_half = [&](int i0, bf16x8 (&fa)[4], bf16x8 (&fb)[k2NBT], auto fresh) {
+    const f32x4v zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < k2NBT; ++j)
-        acc[i0 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], acc[i0 + i][j], 0, 0, 0);
+        acc[i0 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], decltype(fresh)::value ? zero : acc[i0 + i][j],
+                                                                   0, 0, 0);
   };
   int step = 0;
-  auto do_step = [&]() {
+  auto do_step = [&](auto fresh) {
     __builtin_amdgcn_sched_barrier(0);
     read_a(step, 0, 4, fa_hi);
-    mfma_half(0, fa_lo, fb0);
+    mfma_half(0, fa_lo, fb0, fresh);
     pair_reads<2, 4>();
     __builtin_amdgcn_sched_barrier(0);
     read_a(step, 1, 0, fa_lo);
     read_b(step, 1, fb1);
-    mfma_half(4, fa_hi, fb0);
+    mfma_half(4, fa_hi, fb0, fresh);
     pair_reads<2, 8>();
     __builtin_amdgcn_sched_barrier(0);
     read_a(step, 1, 4, fa_hi);
-    mfma_half(0, fa_lo, fb1);
+    mfma_half(0, fa_lo, fb1, std::false_type{});
     pair_reads<2, 4>();
     __builtin_amdgcn_sched_barrier(0);
     // This wave has read all it needs of slab `step` and its share of slab step+1 has landed; after
@@ -697,7 +701,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     read_b(step + 1, 0, fb0);
 #pragma unroll
     for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
-    mfma_half(4, fa_hi, fb1);
+    mfma_half(4, fa_hi, fb1, std::false_type{});
     pair_reads<1, 8>();
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
@@ -710,15 +714,10 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   };
 
   for (int vt = vt0; vt < vt1; ++vt) {
-    for (int kt = 0; kt < nk; ++kt) do_step();
+    do_step(std::true_type{});
+    for (int kt = 1; kt < nk; ++kt) do_step(std::false_type{});
     const int v0 = vt * k2BV;
     fold_tile16<ENT, AMAX>(acc, st, tx, tgt, v0 + wave_v * kWaveV, g, v0 + k2BV > a.V, a.V, a.scale);
-#pragma unroll
-    for (int i = 0; i < k2NBV; ++i)
-#pragma unroll
-      for (int j = 0; j < k2NBT; ++j)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no request may outlive the workgroup's LDS
 
