@@ -30,7 +30,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # belongs to the seeded lengths of make_config2 (2356 valid rows).
 TRAFFIC_ROW_MASKED = 716.6e6 + 0.13e6
 TRAFFIC_ROW_ALL = 1245.4e6 + 0.13e6
-TRAFFIC_FUSED_CFG3 = 1848e6 + 7.8e6
+TRAFFIC_FUSED_CFG3 = 1826e6 + 6.8e6
 
 
 def log(*a):
