@@ -103,3 +103,13 @@ def test_check_maps_codes_to_exceptions():
         _lib.check(-4)
     assert e.value.code == -4
     _lib.check(0)
+
+
+def test_header_is_plain_c():
+    """The boundary is a C ABI: the header must compile as C99 on its own, with no C++ or HIP types."""
+    import subprocess
+    hdr = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "tome_logprob.h")
+    src = '#include "%s"\nint main(void) { return tome_abi_version() == TOME_ABI_VERSION ? 0 : 1; }\n' % hdr
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only", "-x", "c", "-"],
+                       input=src, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr

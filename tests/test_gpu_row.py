@@ -169,3 +169,43 @@ def test_fused_log_softmax_full_matrix(dev, dtype, rows, V, T):
             lse_b = oracle.bf16_to_f32(oracle.bf16_round(oracle.lse_rows(bits, 1.0).astype(np.float32)))
             expected = oracle.bf16_to_f32(oracle.bf16_round(oracle.bf16_to_f32(bits) - lse_b[:, None]))
             assert np.abs(oracle.bf16_to_f32(got) - expected).max() < 5e-3
+
+
+def test_entry_points_replay_correctly_from_a_hip_graph(dev):
+    """Callers that capture their step as a HIP graph: the row kernel (with its split + combine launches) and
+    the fused path (compaction, main and combine kernels, device-side schedule) record no memsets and keep
+    no state, so replays on changing inputs must equal eager calls on the same inputs."""
+    rng = np.random.default_rng(77)
+    rows, V, n, H, Vf = 24, 20011, 600, 128, 3001
+    x = torch.zeros((rows, V), dtype=torch.float32, device=dev)
+    t = torch.zeros(rows, dtype=torch.int32, device=dev)
+    h = torch.zeros((n, H), dtype=torch.bfloat16, device=dev)
+    w = torch.from_numpy((rng.standard_normal((Vf, H)) * 0.2).astype(np.float32)).to(dev).to(torch.bfloat16)
+    tf = torch.zeros(n, dtype=torch.int32, device=dev)
+    valid = torch.ones(n, dtype=torch.int32, device=dev)
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):                                   # warm-up outside the capture
+        tome_amd.token_logprobs(x, t, 0.9, want_argmax=True)
+        tome_amd.fused_lmhead_logprobs(h, w, tf, 1.1, row_valid=valid, want_entropy=True)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        r_row = tome_amd.token_logprobs(x, t, 0.9, want_argmax=True)
+        r_fused = tome_amd.fused_lmhead_logprobs(h, w, tf, 1.1, row_valid=valid, want_entropy=True)
+    for it in range(3):
+        x.copy_(torch.from_numpy((rng.standard_normal((rows, V)) * 2).astype(np.float32)))
+        t.copy_(torch.from_numpy(rng.integers(0, V, rows).astype(np.int32)))
+        h.copy_(torch.from_numpy(rng.standard_normal((n, H)).astype(np.float32)).to(torch.bfloat16))
+        tf.copy_(torch.from_numpy(rng.integers(0, Vf, n).astype(np.int32)))
+        valid.copy_(torch.from_numpy((rng.random(n) < 0.3 + 0.3 * it).astype(np.int32)))   # the valid count changes per replay
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [r_row.lp.clone(), r_row.argmax.clone(), r_fused.lp.clone(), r_fused.entropy.clone()]
+        e_row = tome_amd.token_logprobs(x, t, 0.9, want_argmax=True)
+        e_fused = tome_amd.fused_lmhead_logprobs(h, w, tf, 1.1, row_valid=valid, want_entropy=True)
+        torch.cuda.synchronize()
+        for a, b in zip(got, [e_row.lp, e_row.argmax, e_fused.lp, e_fused.entropy]):
+            assert torch.equal(a, b)
+        (h.float() @ w.float().T).sum().item()                       # unrelated eager work between replays
