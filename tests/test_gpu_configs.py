@@ -57,6 +57,16 @@ def test_config2_full_size(dev):
     np.testing.assert_allclose(lp.cpu().numpy()[sample], oracle.logprob_rows(bits, t, 1.0), atol=1e-4, rtol=0)
     np.testing.assert_allclose(full.entropy.view(-1).cpu().numpy()[sample], oracle.entropy_rows(bits, 1.0), atol=1e-4, rtol=0)
     np.testing.assert_array_equal(full.argmax.view(-1).cpu().numpy()[sample], oracle.argmax_rows(bits))
+    # the sampler over the same 4096 rows (streaming variant: rows too long to keep in registers): the greedy
+    # id is the spike, the drawn id is a candidate, its log-prob is the row kernel's, candidates match the oracle
+    us = torch.rand(G * L, device=dev, generator=g)
+    s = tome_amd.sample_tokens(flat, 1.0, 20, uniforms=us, want_topk=True)
+    assert torch.equal(s.argmax, want_amax) and torch.equal(s.topk_idx[:, 0], want_amax)
+    assert (s.topk_idx == s.token[:, None]).any(dim=1).all()
+    assert (s.topk_logit[:, :-1] >= s.topk_logit[:, 1:]).all()
+    torch.testing.assert_close(s.lp, tome_amd.token_logprobs(flat, s.token, 1.0).lp, atol=2e-6, rtol=0)
+    want_idx, _ = oracle.top_k_rows(bits, 20)
+    np.testing.assert_array_equal(s.topk_idx.cpu().numpy()[sample], want_idx)
 
 
 def _sample_stats(hidden2d, weight, targets, T, sample, dev):
