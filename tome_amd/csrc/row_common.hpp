@@ -50,9 +50,9 @@ __device__ __forceinline__ float max_of(const float (&x)[N]) {
   return m;
 }
 
-// Fold N values of load unit `unit` into a lane's state.
+// Fold N values of load unit `unit` into a lane's state; returns the unit's maximum.
 template <int N, bool ENT, bool AMAX>
-__device__ __forceinline__ void absorb(RowStat& st, const float (&x)[N], int unit, float scale) {
+__device__ __forceinline__ float absorb(RowStat& st, const float (&x)[N], int unit, float scale) {
   const float cm = max_of<N>(x);
   const float mx_new = fmaxf(st.mx, cm);
   if constexpr (AMAX) st.bi = (cm > st.mx) ? unit : st.bi;
@@ -69,6 +69,7 @@ __device__ __forceinline__ void absorb(RowStat& st, const float (&x)[N], int uni
   st.mx = mx_new;
   st.s = s;
   if constexpr (ENT) st.w = w;
+  return cm;
 }
 
 // Workgroup reduction of the per-lane states; the result is valid in every lane of wave 0.

@@ -12,16 +12,20 @@
 // (descending; equal logits by ascending token id).  MLX's own random stream cannot be matched.
 //
 // A row is shared by `splits` workgroups (decode batches are a few dozen rows: one workgroup per row
-// would leave most of the chip idle), each making two passes over its range of the row (the second
-// comes from L2 / MALL for decode-sized batches):
-//   1. online (max, sum 2^(y-m)) for the full-vocabulary lse, and every lane's own largest element;
-//      the k-th largest of the 256 lane maxima is a lower bound `theta` of the k-th largest logit;
-//   2. every element >= theta goes to a candidate buffer in LDS (typically k + a few entries).
+// would leave most of the chip idle).  Each computes, over its range of the row,
+//   * the online (max, sum 2^(y-m)) for the full-vocabulary lse and every lane's own largest element;
+//   * a lower bound `theta` of the k-th largest logit: the k-th largest of the lane maxima (four waves,
+//     each extracting its ceil(k/4) largest);
+//   * every element >= theta, as a candidate in an LDS buffer (typically k + a few entries).
+// Short ranges (a lane owns <= 8 load units) are loaded once and kept in registers for the candidate
+// scan.  Long ranges are streamed once: theta comes from the lanes' first units, is renewed after a
+// quarter of the range, and candidates are collected as the row goes by; only when the buffer overflows
+// is the range scanned a second time with the bound from all of it.
 // Candidates are 64-bit keys (order-preserving image of the float, then ~index), so there are no
 // ties and "the top k" is unique.  A buffer overflow (adversarial orderings only) raises theta to
-// the k-th largest of what was kept - still a lower bound - and repeats pass 2.  The final k are
-// rank-sorted by one wave.  With splits > 1 every workgroup leaves its k keys and its (max, sum)
-// in the workspace and row_sample_combine_kernel selects among the splits * k keys and draws.
+// the k-th largest of what was kept - still a lower bound - and rescans.  The final k are ranked by
+// counting.  With splits > 1 every workgroup leaves its k keys and its (max, sum) in the workspace
+// and row_sample_combine_kernel selects among the splits * k keys and draws.
 #include "row_common.hpp"
 
 namespace tome {
@@ -241,6 +245,20 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
   // single elements after the last whole unit: lane 0 of the last split
   const int n_tail = split == a.splits - 1 ? (int)(a.V - n_units * kVec) : 0;
 
+  const bool big_range = (u1 - u0) * kVec + n_tail > kSampCap;
+  if (tid == 0) sh.cnt = 0;  // published by the first barrier below, before any candidate is offered
+  // A candidate: an element at or above the bound (value first, then the whole key).
+  auto offer = [&](float x, int64_t idx, uint64_t thr, float thr_val) {
+    if (x >= thr_val) {
+      const uint64_t key = make_key(x, (uint32_t)idx);
+      if (key >= thr) {
+        const int pos = atomicAdd(&sh.cnt, 1);
+        if (pos < kSampCap) sh.a[pos] = key;
+      }
+    }
+  };
+  bool collected = false;  // the streaming variant gathers its candidates during pass 1
+
   // ---- pass 1: full-vocabulary statistics and this lane's own maximum --------------------------
   RowStat st = stat_identity();
   u32x4 cached[CACHED ? kSampCached : 1];
@@ -266,30 +284,71 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
       }
     }
   } else if constexpr (VECTOR) {
+    // Streaming variant: candidates are collected during this one pass.  The k-th largest of the
+    // lanes' maxima over their FIRST units is already a lower bound of the row's k-th largest, so
+    // everything at or above it goes to the buffer as it streams by; after a quarter of the range
+    // the bound is renewed from the maxima so far, which lets far less through (a few hundred
+    // candidates per row in all).
     const u32x4* p = reinterpret_cast<const u32x4*>(row);
-    int64_t u = u0 + tid;
-    for (; u + (kRowUnroll - 1) * kRowWG < u1; u += kRowUnroll * kRowWG) {
-      u32x4 v[kRowUnroll];
+    constexpr int kGroup = kRowUnroll * kRowWG;                    // units per workgroup and iteration
+    const int64_t n_groups = (u1 > u0 ? u1 - u0 : 0) / kGroup;     // iterations in which every lane has all its units
+    uint64_t early = 0;  // ranges that fit the buffer are collected whole
+    float early_val = -INFINITY;
+    auto consume = [&](const u32x4& v, int64_t unit) {
+      float x[kVec];
+      Elem<T>::unpack(v, x);
+      if (absorb<kVec, false, true>(st, x, (int)unit, a.scale) >= early_val) {
 #pragma unroll
-      for (int q = 0; q < kRowUnroll; ++q) v[q] = p[u + q * kRowWG];
+        for (int i = 0; i < kVec; ++i) offer(x[i], unit * kVec + i, early, early_val);
+      }
+    };
+    auto renew_bound = [&]() {
+      early = bound_from_lane_maxima(sh, st.bi != 0x7fffffff ? st.mx : -INFINITY, k);
+      early_val = early == 0 ? -INFINITY : key_float((uint32_t)(early >> 32));
+    };
+    int64_t g0 = 0;
+    if (n_groups > 0 && big_range) {  // first iteration: statistics, then the bound, then its candidates
+      u32x4 first[kRowUnroll];
+#pragma unroll
+      for (int q = 0; q < kRowUnroll; ++q) first[q] = p[u0 + tid + q * kRowWG];
 #pragma unroll
       for (int q = 0; q < kRowUnroll; ++q) {
         float x[kVec];
-        Elem<T>::unpack(v[q], x);
-        absorb<kVec, false, true>(st, x, (int)(u + q * kRowWG), a.scale);
+        Elem<T>::unpack(first[q], x);
+        absorb<kVec, false, true>(st, x, (int)(u0 + tid + q * kRowWG), a.scale);
       }
+      renew_bound();  // its barriers also publish sh.cnt == 0
+#pragma unroll
+      for (int q = 0; q < kRowUnroll; ++q) {
+        float x[kVec];
+        Elem<T>::unpack(first[q], x);
+        if (max_of<kVec>(x) >= early_val) {
+#pragma unroll
+          for (int i = 0; i < kVec; ++i) offer(x[i], (u0 + tid + q * kRowWG) * kVec + i, early, early_val);
+        }
+      }
+      g0 = 1;
+    } else {
+      __syncthreads();  // sh.cnt == 0 is visible
     }
-    for (; u < u1; u += kRowWG) {
-      float x[kVec];
-      Elem<T>::unpack(p[u], x);
-      absorb<kVec, false, true>(st, x, (int)u, a.scale);
+    const int64_t g_renew = n_groups >= 8 && big_range ? 1 + (n_groups - 1) / 4 : n_groups;
+    for (int64_t gi = g0; gi < n_groups; ++gi) {
+      if (gi == g_renew) renew_bound();  // uniform: every lane runs the same iterations
+      u32x4 v[kRowUnroll];
+#pragma unroll
+      for (int q = 0; q < kRowUnroll; ++q) v[q] = p[u0 + gi * kGroup + tid + q * kRowWG];
+#pragma unroll
+      for (int q = 0; q < kRowUnroll; ++q) consume(v[q], u0 + gi * kGroup + tid + q * kRowWG);
     }
+    for (int64_t u = u0 + n_groups * kGroup + tid; u < u1; u += kRowWG) consume(p[u], u);
     if (tid == 0) {
       for (int e = 0; e < n_tail; ++e) {
         float x[1] = {Elem<T>::load1(row + n_units * kVec + e)};
         absorb<1, false, true>(st, x, (int)(n_units + e), a.scale);
+        offer(x[0], n_units * kVec + e, early, early_val);
       }
     }
+    collected = true;
   } else {
     for (int64_t u = u0 + tid; u < u1; u += kRowWG) {
       float x[1] = {Elem<T>::load1(row + u)};
@@ -320,29 +379,31 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
     }
     lane_key = make_key(st.mx, (uint32_t)idx);
   }
-  if (tid == 0) sh.cnt = 0;
-  const RowStat tot = block_reduce(st, a.scale, sh.red);  // valid in wave 0
+  const RowStat tot = block_reduce(st, a.scale, sh.red);  // valid in wave 0; its barrier also ends the offers of pass 1
+
+  int m = 0;
+  bool scan = true;
+  if (collected) {
+    const int offered = sh.cnt;
+    if (offered <= kSampCap) {
+      m = offered;
+      scan = false;
+    } else {  // the early bound let too much through: fall back to the bound from the whole range and rescan
+      __syncthreads();
+      if (tid == 0) sh.cnt = 0;
+    }
+  }
 
   // ---- theta: k-th largest lane maximum (ranges that fit the buffer skip the bound) --------------
   uint64_t theta = 0;
-  if ((u1 - u0) * kVec + n_tail > kSampCap) {
-    theta = bound_from_lane_maxima(sh, lane_key != 0 ? st.mx : -INFINITY, k);
-  }
+  if (scan && big_range) theta = bound_from_lane_maxima(sh, lane_key != 0 ? st.mx : -INFINITY, k);
+  else if (scan && collected) __syncthreads();
 
   // ---- pass 2: collect every element >= theta ---------------------------------------------------
-  // sh.cnt is zero here: cleared before the reduction's barrier above, and again after an overflow.
-  int m = 0;
-  for (;;) {
+  // sh.cnt is zero here: cleared before the first barrier, and again after an overflow.
+  while (scan) {
     const float theta_val = theta == 0 ? -INFINITY : key_float((uint32_t)(theta >> 32));
-    auto offer = [&](float x, int64_t idx) {
-      if (x >= theta_val) {
-        const uint64_t key = make_key(x, (uint32_t)idx);
-        if (key >= theta) {
-          const int pos = atomicAdd(&sh.cnt, 1);
-          if (pos < kSampCap) sh.a[pos] = key;
-        }
-      }
-    };
+    auto offer2 = [&](float x, int64_t idx) { offer(x, idx, theta, theta_val); };
     if constexpr (CACHED) {
       // Opaque to the optimiser, so that the keys and element indices below are formed where they are
       // used (rarely) instead of being hoisted out of the retry loop into a hundred live registers.
@@ -358,12 +419,12 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
           Elem<T>::unpack(cached[q], x);
           if (max_of<kVec>(x) >= theta_val) {
 #pragma unroll
-            for (int i = 0; i < kVec; ++i) offer(x[i], first_elem + (uint32_t)(q * kRowWG * kVec + i));
+            for (int i = 0; i < kVec; ++i) offer2(x[i], first_elem + (uint32_t)(q * kRowWG * kVec + i));
           }
           __builtin_amdgcn_sched_barrier(0);
         }
       if (tid == 0)
-        for (int e = 0; e < n_tail; ++e) offer(Elem<T>::load1(row + n_units * kVec + e), n_units * kVec + e);
+        for (int e = 0; e < n_tail; ++e) offer2(Elem<T>::load1(row + n_units * kVec + e), n_units * kVec + e);
     } else if constexpr (VECTOR) {
       const u32x4* p = reinterpret_cast<const u32x4*>(row);
       int64_t u = u0 + tid;
@@ -377,7 +438,7 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
           Elem<T>::unpack(v[q], x);
           if (max_of<kVec>(x) >= theta_val) {
 #pragma unroll
-            for (int i = 0; i < kVec; ++i) offer(x[i], (u + q * kRowWG) * kVec + i);
+            for (int i = 0; i < kVec; ++i) offer2(x[i], (u + q * kRowWG) * kVec + i);
           }
         }
       }
@@ -386,13 +447,13 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
         Elem<T>::unpack(p[u], x);
         if (max_of<kVec>(x) >= theta_val) {
 #pragma unroll
-          for (int i = 0; i < kVec; ++i) offer(x[i], u * kVec + i);
+          for (int i = 0; i < kVec; ++i) offer2(x[i], u * kVec + i);
         }
       }
       if (tid == 0)
-        for (int e = 0; e < n_tail; ++e) offer(Elem<T>::load1(row + n_units * kVec + e), n_units * kVec + e);
+        for (int e = 0; e < n_tail; ++e) offer2(Elem<T>::load1(row + n_units * kVec + e), n_units * kVec + e);
     } else {
-      for (int64_t u = u0 + tid; u < u1; u += kRowWG) offer(Elem<T>::load1(row + u), u);
+      for (int64_t u = u0 + tid; u < u1; u += kRowWG) offer2(Elem<T>::load1(row + u), u);
     }
     __syncthreads();
     const int offered = sh.cnt;
