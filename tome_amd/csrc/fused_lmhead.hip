@@ -9,16 +9,19 @@
 // Decomposition
 //   * The GEMM is computed transposed: MFMA "A" rows are vocab entries (W is [V, H], K
 //     contiguous), MFMA "B" columns are tokens (hidden is [n, H], K contiguous).  In the
-//     32x32 accumulator layout a lane then owns ONE token (lane % 32) and 16 vocab rows per
-//     block, so the softmax row statistics are per-lane registers that persist across the
-//     whole vocab sweep; only lanes l and l^32 share a token and are merged once at the end.
-//   * A workgroup (256 lanes, 4 waves as 2 vocab x 2 token) owns a 128-token tile and a
-//     contiguous range of 256-row vocab tiles.  Per vocab tile it runs the K loop (64-wide
-//     slabs staged through padded LDS, next slab prefetched into registers), then folds the
-//     256x128 accumulator tile into the running (max, sum 2^(y-m), sum y 2^(y-m)) states.
-//   * The vocab axis is split over workgroups so that ~2 workgroups per CU are resident;
-//     each writes one partial per (token, split, vocab-wave) and fused_combine_kernel merges
-//     them deterministically.
+//     accumulator layouts a lane then owns ONE token per block column (lane % 32 with the 32x32
+//     MFMA, lane % 16 with the 16x16 one) and a few vocab rows per block, so the softmax row
+//     statistics are per-lane registers that persist across the whole vocab sweep; the lanes
+//     that share a token are merged once at the end.
+//   * A workgroup owns one token tile and a contiguous range of 256-row vocab tiles.  Per vocab
+//     tile it runs the K loop, then folds the accumulator tile into the running
+//     (max, sum 2^(y-m), sum y 2^(y-m)) states.  Two kernels share this shape:
+//       fused_lmhead_dma_kernel  (H % 64 == 0, more than 128 tokens) 512 lanes, 256 x 256 tile,
+//                                16x16x32 MFMA, K slabs DMA'd into LDS - described at the kernel;
+//       fused_lmhead_kernel      (any H % 8, short batches) 256 lanes, 256 x 128 tile, 32x32x16
+//                                MFMA, 64-wide slabs staged through registers into padded LDS.
+//   * The vocab axis is split over workgroups (fused_schedule); each writes one partial per
+//     (token, split, vocab-wave) and fused_combine_kernel merges them deterministically.
 //   * Masked tokens are compacted first (compact_rows_kernel); token tiles are built from
 //     the compacted index list, so masked rows cost no FLOPs and no HBM traffic.
 #include "common.hpp"
