@@ -487,16 +487,38 @@ __global__ __launch_bounds__(kRowWG) void row_sample_combine_kernel(SampleArgs a
   if (a.row_valid && a.row_valid[r] == 0) return;  // outputs already written by the main kernel
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int k = a.top_k, m = a.splits * k;         // <= 64 * 32 = kSampMergeCap
-  for (int i = tid; i < m; i += kRowWG) sh.a[i] = a.part_keys[r * m + i];
-  __syncthreads();
-  select_top_k(sh, sh.a, sh.b, m, k);
-  if (wave != 0) return;
-  RowStat st = stat_identity();
-  if (lane < a.splits) {
+  const uint64_t* keys = a.part_keys + r * m;      // per split: its k keys in descending order, 0 past the end
+  RowStat st = stat_identity();                    // issued early: overlaps the selection below
+  if (wave == 0 && lane < a.splits) {
     const float2 p = a.part_stat[r * a.splits + lane];
     st.mx = p.x;
     st.s = p.y;
   }
+  // A lower bound of the k-th largest from the heads of the lists: the largest 64 / splits keys of every
+  // split (more than k keys in all); its k-th largest keeps a few dozen of the splits * k keys.
+  if (tid == 0) {
+    sh.thr4[0] = 0;
+    sh.cnt = 0;
+  }
+  __syncthreads();
+  if (m > kRowWG && wave == 0) {
+    const int per = 64 / a.splits;                 // >= 1: splits <= 64
+    const int sp = lane / per, j = lane % per;
+    const uint64_t key = (sp < a.splits && j < k) ? keys[sp * k + j] : 0;
+    const int rank = wave_rank(key, 64);
+    if (key != 0 && rank == k - 1) sh.thr4[0] = key;
+  }
+  __syncthreads();
+  const uint64_t thr = sh.thr4[0];
+  for (int i = tid; i < m; i += kRowWG) {
+    const uint64_t key = keys[i];
+    if (key != 0 && key >= thr) sh.a[atomicAdd(&sh.cnt, 1)] = key;
+  }
+  __syncthreads();
+  const int kept = sh.cnt;
+  __syncthreads();
+  select_top_k(sh, sh.a, sh.b, kept, k);
+  if (wave != 0) return;
   stat_wave_reduce(st, a.scale);
   finish_sample(a, sh, r, st, lane);
 }
