@@ -9,6 +9,7 @@
 namespace tome {
 
 constexpr int kFullWG = 256;
+constexpr int kFullUnroll = 4;
 
 struct FullArgs {
   const void* in;
@@ -58,8 +59,7 @@ __global__ __launch_bounds__(kFullWG) void full_log_softmax_kernel(FullArgs a) {
   if constexpr (VECTOR) {
     const u32x4* src = reinterpret_cast<const u32x4*>(in_row);
     u32x4* dst = reinterpret_cast<u32x4*>(out_row);
-    for (int64_t u = u0 + threadIdx.x; u < u1; u += kFullWG) {
-      const u32x4 v = src[u];
+    auto convert = [&](const u32x4& v) {
       u32x4 o;
       if constexpr (BF16) {
         o.x = sub_pack_bf16(v.x, a.inv_temp, lse_t);
@@ -72,8 +72,17 @@ __global__ __launch_bounds__(kFullWG) void full_log_softmax_kernel(FullArgs a) {
         o.z = __float_as_uint(__fsub_rn(__fmul_rn(__uint_as_float(v.z), a.inv_temp), lse_t));
         o.w = __float_as_uint(__fsub_rn(__fmul_rn(__uint_as_float(v.w), a.inv_temp), lse_t));
       }
-      __builtin_nontemporal_store(o, dst + u);
+      return o;
+    };
+    int64_t u = u0 + threadIdx.x;
+    for (; u + (kFullUnroll - 1) * kFullWG < u1; u += kFullUnroll * kFullWG) {  // several 16-byte loads in flight per lane
+      u32x4 v[kFullUnroll];
+#pragma unroll
+      for (int q = 0; q < kFullUnroll; ++q) v[q] = __builtin_nontemporal_load(src + u + q * kFullWG);
+#pragma unroll
+      for (int q = 0; q < kFullUnroll; ++q) __builtin_nontemporal_store(convert(v[q]), dst + u + q * kFullWG);
     }
+    for (; u < u1; u += kFullWG) __builtin_nontemporal_store(convert(src[u]), dst + u);
     if (chunk == a.chunks - 1 && threadIdx.x == 0)
       for (int64_t e = n_units * kVec; e < a.V; ++e) scalar_elem(e);
   } else {
