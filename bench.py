@@ -31,6 +31,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 TRAFFIC_ROW_MASKED = 716.6e6 + 0.13e6
 TRAFFIC_ROW_ALL = 1245.4e6 + 0.13e6
 TRAFFIC_FUSED_CFG3 = 1826e6 + 6.8e6
+TRAFFIC_DECODE_64 = 39.4e6 + 0.42e6 + 0.40e6   # sampler: main-kernel fetch, combine fetch, partials written
 
 
 def log(*a):
@@ -307,7 +308,7 @@ def main():
                                     "fp32 logits [64, 151936] (config 1's shape), top_k 20",
                         "rows": decode["rows"], "top_k": decode["top_k"], "vocab": V},
              "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                          "frac": gbs / HBM_PEAK_GBS, "traffic": TRAFFIC_DECODE_64,
                           "kernel": "row_sample_kernel<f32> + row_sample_combine_kernel",
                           "bytes_per_launch": decode["bytes"]}}
         if row is None and fused is None:
