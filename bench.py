@@ -32,6 +32,7 @@ TRAFFIC_ROW_MASKED = 716.6e6 + 0.13e6
 TRAFFIC_ROW_ALL = 1245.4e6 + 0.13e6
 TRAFFIC_FUSED_CFG3 = 1826e6 + 6.8e6
 TRAFFIC_DECODE_64 = 39.4e6 + 0.42e6 + 0.40e6   # sampler: main-kernel fetch, combine fetch, partials written
+TRAFFIC_LORA_06B = 812.1e6 + 763.4e6            # merge kernel: fetch + write (profiles/lora_merge_kernel_qwen3_0.6b_update.txt)
 
 
 def log(*a):
@@ -177,6 +178,47 @@ def bench_decode(dev, steps, warmup):
     return {"rows": rows, "top_k": k, "ms": ms, "bytes": rows * V * 4}
 
 
+def bench_lora(dev, steps, warmup):
+    """One UpdateWeights (mlx-impl/node.py:102-164) at Qwen3-0.6B's shape: 28 layers x (qkv_proj [4096, 1024],
+    gate_up_proj [6144, 1024], down_proj [1024, 3072]), rank 8, scale 2.5 - 84 merges, one C-ABI call.
+    Algorithmic bytes: every base weight read once and every policy weight written once."""
+    import ctypes
+    import torch
+    import tome_amd
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    layers, rank = 28, 8
+    shapes = [(4096, 1024), (6144, 1024), (1024, 3072)]
+    g = torch.Generator(device=dev).manual_seed(99)
+    keep, n_bytes = [], 0
+    jobs = (_lib.TomeLoraJob * (layers * len(shapes)))()
+    for i in range(layers * len(shapes)):
+        rows, cols = shapes[i % len(shapes)]
+        base = (torch.randn((rows, cols), device=dev, generator=g) * 0.02).to(torch.bfloat16)
+        out = torch.empty_like(base)
+        a = (torch.randn((rank, cols), device=dev, generator=g) * 0.05).to(torch.bfloat16)
+        b = (torch.randn((rows, rank), device=dev, generator=g) * 0.05).to(torch.bfloat16)
+        keep += [base, out, a, b]
+        j = jobs[i]
+        j.base, j.out, j.lora_a, j.lora_b = base.data_ptr(), out.data_ptr(), a.data_ptr(), b.data_ptr()
+        j.rows, j.cols, j.rank, j.base_stride, j.out_stride, j.scale = rows, cols, rank, cols, cols, 2.5
+        n_bytes += rows * cols * 4
+    jp = ctypes.cast(jobs, ctypes.c_void_p)
+    ws_bytes = lib.tome_lora_merge_workspace(jp, len(jobs))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def step():
+        _lib.check(lib.tome_lora_merge(jp, len(jobs), ws.data_ptr(), ws_bytes, stream))
+    step()
+    torch.cuda.synchronize()
+    base, out, a, b = keep[:4]                      # gate on what is timed: the first merge against fp32 torch
+    want = base.float() + 2.5 * (b.float() @ a.float())
+    assert (out.float() - want).abs().max().item() <= 2.0 ** -8 * want.abs().max().item() + 1e-3
+    ms, wall = time_steps(step, steps, warmup)
+    return {"ms": ms, "wall_ms": wall, "bytes": n_bytes, "jobs": len(jobs), "rank": rank}
+
+
 def cpu_baseline(sample_rows=256, budget_s=12.0):
     """NumPy fp32 restatement of local_compute_logprobs (mlx-impl/node.py:400-404) on a bounded
     sample of the config-2 workload: `sample_rows` rows of bf16 logits, upcast included."""
@@ -221,7 +263,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["row", "fused", "decode"], default=None)
+    ap.add_argument("--only", choices=["row", "fused", "decode", "lora"], default=None)
     ap.add_argument("--row-variant", choices=["both", "mask", "all"], default="both",
                     help="time config 2 with its padding mask, without it, or both (profiling runs pick one)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -254,6 +296,7 @@ def main():
     # still settle (a few tens of milliseconds of back-to-back launches are needed for that)
     fused = bench_fused(dev, max(5, args.steps // 2), max(2, args.warmup // 2)) if args.only in (None, "fused") else None
     decode = bench_decode(dev, args.steps, args.warmup) if args.only in (None, "decode") else None
+    lora = bench_lora(dev, max(5, args.steps // 4), max(2, args.warmup // 4)) if args.only in (None, "lora") else None
     cpu = None if args.no_cpu else cpu_baseline()
 
     line = {
@@ -316,6 +359,19 @@ def main():
                          "roofline": d["roofline"]})
         else:
             line["decode_sampler"] = d
+    if lora is not None:
+        gbs = lora["bytes"] / (lora["ms"] * 1e-3) / 1e9
+        d = {"value": lora["jobs"] / (lora["ms"] * 1e-3), "unit": "weight matrices merged/s", "ms_per_step": lora["ms"],
+             "dtype": "bf16",
+             "config": {"workload": "UpdateWeights at Qwen3-0.6B's shape: 28 layers x (qkv, gate_up, down), LoRA rank 8",
+                        "matrices": lora["jobs"], "rank": lora["rank"]},
+             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                          "traffic": TRAFFIC_LORA_06B, "kernel": "lora_merge_kernel<1>", "bytes_per_launch": lora["bytes"]}}
+        if row is None and fused is None and decode is None:
+            line.update({"value": d["value"], "unit": d["unit"], "ms_per_step": d["ms_per_step"], "config": d["config"],
+                         "roofline": d["roofline"], "dtype": "bf16"})
+        else:
+            line["lora_merge"] = d
     if cpu is not None:
         line["cpu_baseline"] = cpu
     print(json.dumps(line), flush=True)

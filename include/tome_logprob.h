@@ -151,6 +151,54 @@ int tome_grpo_dual(const void* hidden, const void* w_policy, const void* w_ref, 
                    float* out_lp, float* out_ref_lp, float* out_k3, float* out_entropy,
                    void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- GRPO policy + reference pass as the reference's two models produce it ---------
+ * The reference keeps two models, `self.model` (policy) and `self.reference_model`
+ * (mlx-impl/node.py:65-66,443); UpdateWeights changes attention and MLP weights only
+ * (node.py:134-151), so the two differ in their final HIDDEN STATES while the final norm
+ * (mlx-impl/model.py:536) and the lm_head (model.py:537-538) stay shared.  This entry
+ * takes one hidden-state matrix per model - both [n_tokens, H] bf16 with the same stride -
+ * and one or two lm_head weights (w_ref may equal w_policy); `norm_weight` is nullable
+ * and, when given, both inputs are pre-norm states as in tome_norm_lmhead_logprob.
+ * Outputs as tome_grpo_dual.
+ */
+size_t tome_grpo_pair_workspace(int64_t n_tokens, int64_t H, int64_t V, int with_norm);
+int tome_grpo_pair(const void* hidden_policy, const void* hidden_ref, const void* norm_weight,
+                   float norm_eps, const void* w_policy, const void* w_ref, int64_t n_tokens,
+                   int64_t H, int64_t V, int64_t hidden_stride, int64_t weight_stride,
+                   const int32_t* targets, const int32_t* row_valid, float temperature,
+                   float* out_lp, float* out_ref_lp, float* out_k3, float* out_entropy,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- LoRA merge: the arithmetic of UpdateWeights -----------------------------------
+ * Replaces `delta_W = scale * (lora_B @ lora_A)` (mlx-impl/node.py:128) and
+ * `policy_W = base_W + delta_W` (node.py:137,146,149,151) for a batch of weight matrices in
+ * one launch.  Everything is bf16; intermediates are rounded where the reference's array
+ * expressions round them:  out = bf16(base + bf16(bf16(scale) * bf16(lora_B @ lora_A))),
+ * the product accumulated in fp32.  A job with lora_a == NULL (and lora_b == NULL) writes
+ * bf16(base + 0): the q/k/v slices the reference fills with zeros (node.py:142-145).
+ * `jobs` is a HOST array, consumed before the call returns.  The workspace (device memory,
+ * 16-byte aligned, size from tome_lora_merge_workspace for the same jobs) receives the job
+ * table and each lora_A transposed; it must stay untouched until the launches have run.
+ *   base, out     [rows, cols] bf16, strides in elements (>= cols, multiples of 8), 16-byte
+ *                 aligned; out may be base itself (in place), any other overlap is undefined
+ *   lora_a        [rank, cols] bf16 contiguous (LayerUpdate.lora_A, inference.proto:71)
+ *   lora_b        [rows, rank] bf16 contiguous, 16-byte aligned (lora_B, inference.proto:72)
+ *   rank          multiple of 8, 8..128;  cols multiple of 8
+ *   scale         LayerUpdate.lora_scale; the caller maps 0 to 1.0 as node.py:127 does
+ */
+typedef struct TomeLoraJob {
+  const void* base;
+  void* out;
+  const void* lora_a;
+  const void* lora_b;
+  int64_t rows, cols, rank, base_stride, out_stride;
+  float scale;
+  int32_t reserved;
+} TomeLoraJob;
+size_t tome_lora_merge_workspace(const TomeLoraJob* jobs, int64_t n_jobs);
+int tome_lora_merge(const TomeLoraJob* jobs, int64_t n_jobs, void* workspace, size_t workspace_bytes,
+                    void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -62,6 +62,18 @@ Pinning (tests/test_oracle.py):
                             kept with its log-prob in Rollout and dropped in Judge,
                             the first token never checked in Rollout, the
                             max_tokens cut, eos / 0 fed to finished rows.
+  lora_merge_bf16 / update_weights  node.py:102-164.  The mathematics base + scale * B @ A
+                            is pinned by closed forms (zero A -> the base bit for bit,
+                            rank-1 outer product, B selecting rows of A, linearity in
+                            scale on exactly representable inputs), brute-force loops
+                            with math.fsum, and numpy's float64 matmul; the
+                            bookkeeping (last update wins, scale 0 -> 1.0, qkv_proj
+                            over q/k/v, missing q/k/v slices revert to the base,
+                            non-cumulative, untouched layers kept) by known-answer
+                            tests on a two-layer toy model.  WHERE MLX rounds to bf16
+                            (matmul output, scalar cast to bf16 before the multiply,
+                            the sum) is restated from MLX's published semantics:
+                            parity unpinned by the reference's tests.
   process_ref_logprobs_batched  known-answer tests on a stub model
                             (alignment, empty completion, temperature 0,
                             chunking, padding id 0) and the length contract of
@@ -79,6 +91,7 @@ __all__ = [
     "argmax_rows", "k3", "lmhead_logits64", "lmhead_stats", "full_log_softmax64",
     "local_compute_logprobs_f32", "fused_log_softmax_f32", "process_ref_logprobs_batched",
     "rms_norm64", "rms_norm_bf16", "top_k_rows", "sample_top_k", "rollout_decode", "judge_decode",
+    "lora_merge64", "lora_merge_bf16", "update_weights",
 ]
 
 
@@ -336,6 +349,103 @@ def process_ref_logprobs_batched(prompts: Sequence, results: Sequence, G: int,
             results[p_idx].completions[g].ref_log_probs.extend(lps.tolist())  # node.py:458
             num_toks += len(c_toks)
     return num_toks
+
+
+# --------------------------------------------------------------------------
+# UpdateWeights (mlx-impl/node.py:102-164); weights are bf16 bit patterns (uint16)
+# --------------------------------------------------------------------------
+def lora_merge64(base: np.ndarray, lora_a: np.ndarray, lora_b: np.ndarray, scale: float) -> np.ndarray:
+    """base_W + scale * (lora_B @ lora_A) in fp64 on exactly-upcast inputs, no intermediate rounding:
+    the mathematical statement of node.py:128,137.  lora_a [rank, in], lora_b [out, rank]."""
+    return to_f64(base) + float(scale) * (to_f64(lora_b) @ to_f64(lora_a))
+
+
+def _bf16_of_f64(x: np.ndarray) -> np.ndarray:
+    """float64 -> bf16 bit patterns, one correct rounding (ties to even).  Going through float32
+    first would round twice; instead round the float64 significand directly."""
+    x = np.ascontiguousarray(x, dtype=np.float64)
+    f32 = x.astype(np.float32)
+    bits = bf16_round(f32)
+    # repair double rounding: compare against both neighbours in exact float64 arithmetic
+    up = bf16_to_f32(bits).astype(np.float64)
+    lo_bits = np.where(up > x, _bf16_step(bits, -1), bits)
+    hi_bits = _bf16_step(lo_bits, +1)
+    lo = bf16_to_f32(lo_bits).astype(np.float64)
+    hi = bf16_to_f32(hi_bits).astype(np.float64)
+    with np.errstate(invalid="ignore", over="ignore"):
+        d_lo, d_hi = x - lo, hi - x
+    pick_hi = (d_hi < d_lo) | ((d_hi == d_lo) & ((lo_bits & 1) == 1))
+    out = np.where(pick_hi, hi_bits, lo_bits).astype(np.uint16)
+    special = ~np.isfinite(x) | ~np.isfinite(hi) | ~np.isfinite(lo) | (x == 0)
+    return np.where(special, bits, out).astype(np.uint16)
+
+
+def _bf16_step(bits: np.ndarray, direction: int) -> np.ndarray:
+    """Next bf16 value towards +inf (direction +1) or -inf (-1), on bit patterns of finite values."""
+    b = bits.astype(np.int32)
+    neg = (b & 0x8000) != 0
+    mag = b & 0x7FFF
+    if direction > 0:
+        mag2 = np.where(neg, mag - 1, mag + 1)
+        flip = neg & (mag == 0)
+        out = np.where(flip, 0x0001, np.where(neg, 0x8000 | mag2, mag2))
+    else:
+        mag2 = np.where(neg, mag + 1, mag - 1)
+        flip = (~neg) & (mag == 0)
+        out = np.where(flip, 0x8001, np.where(neg, 0x8000 | mag2, mag2))
+    return (out & 0xFFFF).astype(np.uint16)
+
+
+def lora_merge_bf16(base: np.ndarray, lora_a, lora_b, scale: float) -> np.ndarray:
+    """The same with the roundings of the reference's bf16 array expressions, bit patterns in and out:
+    ``delta_W = scale * (lora_B @ lora_A)`` (node.py:128) is a bf16 matmul (exact products, wide
+    accumulation, ONE rounding to bf16) times a Python scalar that MLX first casts to the array's
+    dtype, the product rounded to bf16; ``base_W + delta_W`` (node.py:137) rounds once more.
+    ``lora_a is None`` stands for the ``mx.zeros_like`` deltas of node.py:143-145."""
+    b64 = to_f64(base)
+    if lora_a is None:
+        return _bf16_of_f64(b64 + 0.0)
+    d = to_f64(_bf16_of_f64(to_f64(lora_b) @ to_f64(lora_a)))
+    s = to_f64(bf16_round(np.float32(scale).reshape(1)))[0]
+    d2 = to_f64(_bf16_of_f64(s * d))
+    return _bf16_of_f64(b64 + d2)
+
+
+def update_weights(policy: list, reference: list, updates: Sequence, *, num_heads: int, num_kv_heads: int,
+                   head_dim: int) -> int:
+    """node.py:114-151 on dict models: ``policy[i]`` / ``reference[i]`` map ``"self_attn.qkv_proj"``,
+    ``"mlp.gate_up_proj"``, ``"mlp.down_proj"`` to bf16 bit patterns [out, in]; ``updates`` carry
+    ``layer_idx, param_name, lora_A, lora_B`` (bytes), ``shape_A, shape_B, lora_scale``
+    (scheduler/proto/inference.proto:68-76).  Mutates ``policy``; returns the matrices rebuilt."""
+    layer_deltas: dict = {}
+    for up in updates:                                                    # node.py:117-130
+        if not up.lora_A or not up.lora_B:
+            continue
+        a = np.frombuffer(up.lora_A, dtype=np.uint16).reshape(list(up.shape_A))
+        b = np.frombuffer(up.lora_B, dtype=np.uint16).reshape(list(up.shape_B))
+        scale = up.lora_scale if up.lora_scale != 0.0 else 1.0
+        layer_deltas.setdefault(up.layer_idx, {})[up.param_name] = (a, b, scale)
+    rebuilt = 0
+    for layer_idx, deltas in layer_deltas.items():                        # node.py:132-151
+        ref, tgt = reference[layer_idx], policy[layer_idx]
+        base = ref["self_attn.qkv_proj"]
+        if "self_attn.qkv_proj" in deltas:
+            tgt["self_attn.qkv_proj"] = lora_merge_bf16(base, *deltas["self_attn.qkv_proj"])
+            rebuilt += 1
+        elif any(k in deltas for k in ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj")):
+            q_size, k_size = num_heads * head_dim, num_kv_heads * head_dim
+            parts = []
+            for name, lo, hi in (("self_attn.q_proj", 0, q_size), ("self_attn.k_proj", q_size, q_size + k_size),
+                                 ("self_attn.v_proj", q_size + k_size, base.shape[0])):
+                a, b, sc = deltas.get(name, (None, None, 1.0))
+                parts.append(lora_merge_bf16(base[lo:hi], a, b, sc))
+            tgt["self_attn.qkv_proj"] = np.concatenate(parts, axis=0)
+            rebuilt += 1
+        for name in ("mlp.gate_up_proj", "mlp.down_proj"):
+            if name in deltas:
+                tgt[name] = lora_merge_bf16(ref[name], *deltas[name])
+                rebuilt += 1
+    return rebuilt
 
 
 def _draw(logits_row: np.ndarray, u, temperature: float, top_k: int):

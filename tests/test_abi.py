@@ -94,6 +94,35 @@ def test_argument_checks_run_on_host():
     assert lib.tome_row_sample_workspace(0, 4096, 151936, 20) == 0 and lib.tome_row_sample_workspace(0, 64, 151936, 20) > 0
     dual = lib.tome_grpo_dual(P, P, None, 8, 64, 100, 64, 64, P, None, 1.0, P, P, P, P, None, 0, None)
     assert dual == -1
+    pair = lambda **k: lib.tome_grpo_pair(P, k.get("href", P), k.get("nw", None), k.get("eps", 1e-6), P, k.get("wref", P), 8, 64,
+                                          100, 64, 64, P, None, k.get("T", 1.0), P, k.get("ref_lp", P), P, P, None, 0, None)
+    assert pair(href=None) == -1 and pair(wref=None) == -1 and pair(ref_lp=None) == -1
+    assert pair(href=P + 2) == -6 and pair(nw=P + 8) == -6 and pair(nw=P, eps=-1.0) == -3 and pair(T=0.0) == -5
+    assert pair() == -4
+    assert lib.tome_grpo_pair_workspace(4096, 1024, 151936, 0) == lib.tome_grpo_dual_workspace(4096, 1024, 151936)
+    assert lib.tome_grpo_pair_workspace(4096, 1024, 151936, 1) >= lib.tome_grpo_dual_workspace(4096, 1024, 151936) + 2 * 4096 * 1024 * 2
+
+    def merge(**k):
+        j = _lib.TomeLoraJob()
+        j.base, j.out, j.lora_a, j.lora_b = k.get("base", P), k.get("out", P), k.get("a", P), k.get("b", P)
+        j.rows, j.cols, j.rank = k.get("rows", 32), k.get("cols", 64), k.get("rank", 8)
+        j.base_stride, j.out_stride, j.scale = k.get("bs", 64), k.get("os", 64), k.get("scale", 2.5)
+        jp = ctypes.cast(ctypes.pointer(j), ctypes.c_void_p)
+        if k.get("query"):
+            return lib.tome_lora_merge_workspace(jp, k.get("n", 1))
+        return lib.tome_lora_merge(jp, k.get("n", 1), k.get("ws", P), k.get("wsb", 1 << 20), None)
+    assert merge(n=0) == 0 and merge(n=-1) == -3
+    assert lib.tome_lora_merge(None, 1, None, 0, None) == -1
+    table = 256                                    # the job table, rounded up
+    assert merge(query=True) == table + 64 * 32 * 2
+    assert merge(query=True, rank=40, cols=1024, bs=1024, os=1024) == table + 1024 * 64 * 2
+    assert merge(query=True, a=None, b=None) == table and merge(query=True, rank=12) == 0
+    assert merge(ws=None) == -4 and merge(wsb=100) == -4 and merge(ws=P + 4) == -6
+    assert merge(base=None) == -1 and merge(out=None) == -1 and merge(a=None) == -1 and merge(b=None) == -1
+    assert merge(rows=-1) == -3 and merge(cols=0) == -3 and merge(bs=56) == -3 and merge(os=8) == -3
+    assert merge(rank=0) == -3 and merge(rank=136) == -3 and merge(scale=float("inf")) == -3
+    assert merge(rank=12) == -6 and merge(cols=60, bs=64) == -6 and merge(bs=68) == -6 and merge(base=P + 8) == -6
+    assert merge(b=P + 4) == -6
 
 
 def test_check_maps_codes_to_exceptions():

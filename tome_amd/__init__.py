@@ -15,11 +15,13 @@ from .logprob import (  # noqa: F401
     DecodeStepGraph,
     fused_lmhead_logprobs,
     grpo_dual_logprobs,
+    grpo_pair_logprobs,
     TokenLogprobs,
     SampledTokens,
     DualLogprobs,
 )
 from .decode import rollout_decode, judge_decode  # noqa: F401
+from .weights import LayerUpdate, WeightUpdateResponse, WeightUpdateServicer, apply_weight_update, lora_merge  # noqa: F401
 from .node import Prompt, Completion, PromptRollout, RefLogprobServicer  # noqa: F401
 from .wire import (  # noqa: F401
     PackedRefChunk, pack_ref_work, scatter_ref_logprobs, rollout_response_to_json, rollout_response_from_json,
@@ -28,7 +30,8 @@ from ._lib import TomeError, lib_path, load_library  # noqa: F401
 
 __all__ = [
     "fused_log_softmax", "local_compute_logprobs", "token_logprobs", "sample_tokens", "DecodeStepGraph", "fused_lmhead_logprobs",
-    "grpo_dual_logprobs", "TokenLogprobs", "SampledTokens", "DualLogprobs", "Prompt", "Completion", "PromptRollout",
+    "grpo_dual_logprobs", "grpo_pair_logprobs", "LayerUpdate", "WeightUpdateResponse", "WeightUpdateServicer",
+    "apply_weight_update", "lora_merge", "TokenLogprobs", "SampledTokens", "DualLogprobs", "Prompt", "Completion", "PromptRollout",
     "RefLogprobServicer", "rollout_decode", "judge_decode", "PackedRefChunk", "pack_ref_work", "scatter_ref_logprobs",
     "rollout_response_to_json", "rollout_response_from_json", "TomeError", "lib_path", "load_library",
 ]

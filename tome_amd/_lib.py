@@ -38,7 +38,20 @@ SIGNATURES = {
     "tome_grpo_dual": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_size_t, c_void_p]),
+    "tome_grpo_pair_workspace": (c_size_t, [c_int64, c_int64, c_int64, c_int]),
+    "tome_grpo_pair": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                               c_int64, c_int64, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_size_t, c_void_p]),
+    "tome_lora_merge_workspace": (c_size_t, [c_void_p, c_int64]),
+    "tome_lora_merge": (c_int, [c_void_p, c_int64, c_void_p, c_size_t, c_void_p]),
 }
+
+
+class TomeLoraJob(ctypes.Structure):
+    """``TomeLoraJob`` of include/tome_logprob.h."""
+    _fields_ = [("base", c_void_p), ("out", c_void_p), ("lora_a", c_void_p), ("lora_b", c_void_p),
+                ("rows", c_int64), ("cols", c_int64), ("rank", c_int64), ("base_stride", c_int64),
+                ("out_stride", c_int64), ("scale", c_float), ("reserved", ctypes.c_int32)]
 
 
 class TomeError(RuntimeError):

@@ -27,6 +27,14 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, floa
                                const int32_t* row_valid, float temperature, float* out_lp, float* out_lse,
                                float* out_entropy, int32_t* out_argmax, float* out_ref_lp, float* out_k3,
                                void* workspace, hipStream_t stream);
+hipError_t fused_pair_launch(const void* hidden, const void* hidden_ref, const void* norm_weight, float norm_eps,
+                             const void* w0, const void* w1, int64_t n_tokens, int64_t H, int64_t V,
+                             int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
+                             const int32_t* row_valid, float temperature, float* out_lp, float* out_entropy,
+                             float* out_ref_lp, float* out_k3, void* workspace, hipStream_t stream);
+struct LoraJobHost;
+hipError_t lora_merge_launch(const LoraJobHost* jobs, int n_jobs, void* workspace, hipStream_t stream);
+size_t lora_workspace_bytes(const LoraJobHost* jobs, int n_jobs);
 }  // namespace tome
 
 namespace {
@@ -218,6 +226,72 @@ int tome_grpo_dual(const void* hidden, const void* w_policy, const void* w_ref, 
                                               targets, row_valid, temperature, out_lp, nullptr, out_entropy,
                                               nullptr, out_ref_lp, out_k3, workspace,
                                               static_cast<hipStream_t>(stream)));
+}
+
+size_t tome_grpo_pair_workspace(int64_t n_tokens, int64_t H, int64_t V, int with_norm) {
+  if (n_tokens <= 0 || H <= 0 || V <= 0) return 0;
+  // two partial sets; with a norm weight, one normalised copy per hidden-state matrix
+  return align256(tome::fused_workspace_bytes(n_tokens, H, V, 2, with_norm != 0) +
+                  (with_norm ? align256((size_t)n_tokens * H * 2) : 0));
+}
+
+int tome_grpo_pair(const void* hidden_policy, const void* hidden_ref, const void* norm_weight, float norm_eps,
+                   const void* w_policy, const void* w_ref, int64_t n_tokens, int64_t H, int64_t V,
+                   int64_t hidden_stride, int64_t weight_stride, const int32_t* targets, const int32_t* row_valid,
+                   float temperature, float* out_lp, float* out_ref_lp, float* out_k3, float* out_entropy,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = check_fused(hidden_policy, w_policy, n_tokens, H, V, hidden_stride, weight_stride, targets, temperature);
+  if (rc != TOME_OK || n_tokens == 0) return rc;
+  if (!hidden_ref || !w_ref || !out_lp || !out_ref_lp) return TOME_E_NULL;
+  if (reinterpret_cast<uintptr_t>(w_ref) % 16 != 0 || reinterpret_cast<uintptr_t>(hidden_ref) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(norm_weight) % 16 != 0)
+    return TOME_E_ALIGN;
+  if (norm_weight && (!(norm_eps >= 0.f) || !isfinite(norm_eps))) return TOME_E_SHAPE;
+  const size_t need = tome_grpo_pair_workspace(n_tokens, H, V, norm_weight != nullptr);
+  if (!workspace || workspace_bytes < need) return TOME_E_WORKSPACE;
+  return hip_result(tome::fused_pair_launch(hidden_policy, hidden_ref, norm_weight, norm_eps, w_policy, w_ref, n_tokens,
+                                            H, V, hidden_stride, weight_stride, targets, row_valid, temperature,
+                                            out_lp, out_entropy, out_ref_lp, out_k3, workspace,
+                                            static_cast<hipStream_t>(stream)));
+}
+
+static int check_lora_jobs(const TomeLoraJob* jobs, int64_t n_jobs) {
+  if (n_jobs < 0 || n_jobs > 65536) return TOME_E_SHAPE;
+  if (n_jobs == 0) return TOME_OK;
+  if (!jobs) return TOME_E_NULL;
+  int64_t units = 0;
+  for (int64_t i = 0; i < n_jobs; ++i) {
+    const TomeLoraJob& j = jobs[i];
+    if (!j.base || !j.out) return TOME_E_NULL;
+    if ((j.lora_a == nullptr) != (j.lora_b == nullptr)) return TOME_E_NULL;
+    if (j.rows < 0 || j.cols <= 0 || j.rows > 0x7fffffff - 16 || j.cols > 0x7fffffff - 512) return TOME_E_SHAPE;
+    if (j.base_stride < j.cols || j.out_stride < j.cols || j.base_stride > 0x7fffffff || j.out_stride > 0x7fffffff)
+      return TOME_E_SHAPE;
+    if (j.lora_a && (j.rank < 8 || j.rank > 128)) return TOME_E_SHAPE;
+    if (!isfinite(j.scale)) return TOME_E_SHAPE;
+    if (j.cols % 8 != 0 || j.base_stride % 8 != 0 || j.out_stride % 8 != 0 || (j.lora_a && j.rank % 8 != 0) ||
+        reinterpret_cast<uintptr_t>(j.base) % 16 != 0 || reinterpret_cast<uintptr_t>(j.out) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(j.lora_b) % 16 != 0 || reinterpret_cast<uintptr_t>(j.lora_a) % 2 != 0)
+      return TOME_E_ALIGN;
+    units += ((j.rows + 15) / 16) * ((j.cols + 511) / 512);
+    if (units > 0x7fffffff) return TOME_E_SHAPE;  // one workgroup per unit at most: must fit the grid
+  }
+  return TOME_OK;
+}
+
+size_t tome_lora_merge_workspace(const TomeLoraJob* jobs, int64_t n_jobs) {
+  if (check_lora_jobs(jobs, n_jobs) != TOME_OK || n_jobs == 0) return 0;
+  return tome::lora_workspace_bytes(reinterpret_cast<const tome::LoraJobHost*>(jobs), (int)n_jobs);
+}
+
+int tome_lora_merge(const TomeLoraJob* jobs, int64_t n_jobs, void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = check_lora_jobs(jobs, n_jobs);
+  if (rc != TOME_OK || n_jobs == 0) return rc;
+  const size_t need = tome::lora_workspace_bytes(reinterpret_cast<const tome::LoraJobHost*>(jobs), (int)n_jobs);
+  if (!workspace || workspace_bytes < need) return TOME_E_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return TOME_E_ALIGN;
+  return hip_result(tome::lora_merge_launch(reinterpret_cast<const tome::LoraJobHost*>(jobs), (int)n_jobs, workspace,
+                                            static_cast<hipStream_t>(stream)));
 }
 
 }  // extern "C"

@@ -48,6 +48,13 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
   return (uint16_t)(u >> 16);
 }
 
+// Two floats -> packed bf16 (lo in bits 0..15), round-to-nearest-even: one v_cvt_pk_bf16_f32 on gfx950.
+typedef __bf16 bf16x2_hw __attribute__((ext_vector_type(2)));
+typedef float f32x2_hw __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_hw{lo, hi}, bf16x2_hw));
+}
+
 // ---- wave64 lane exchange --------------------------------------------------------------
 // Steps inside a 16-lane row use DPP (no LDS traffic); the two steps that cross rows go
 // through the LDS crossbar (ds_bpermute via __shfl_xor).  After steps 0..3 every lane of a

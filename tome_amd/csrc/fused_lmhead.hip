@@ -1028,12 +1028,17 @@ static void launch_main(const FusedArgs& a, FusedKind kind, int grid, bool want_
   }
 }
 
-hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, float norm_eps, const void* w0,
-                               const void* w1, int64_t n_tokens, int64_t H, int64_t V, int64_t hidden_stride,
-                               int64_t weight_stride, const int32_t* targets,
-                               const int32_t* row_valid, float temperature, float* out_lp, float* out_lse,
-                               float* out_entropy, int32_t* out_argmax, float* out_ref_lp, float* out_k3,
-                               void* workspace, hipStream_t stream) {
+// One sweep per (hidden, weight) pair: the policy pair always, and a reference pair when a second weight
+// set (`w1`) or a second hidden-state matrix (`hidden_ref`) is given; either may repeat the policy's.
+static hipError_t fused_launch_impl(const void* hidden, const void* hidden_ref, const void* norm_weight,
+                                    float norm_eps, const void* w0, const void* w1, int64_t n_tokens, int64_t H,
+                                    int64_t V, int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
+                                    const int32_t* row_valid, float temperature, float* out_lp, float* out_lse,
+                                    float* out_entropy, int32_t* out_argmax, float* out_ref_lp, float* out_k3,
+                                    void* workspace, hipStream_t stream) {
+  const bool second = w1 != nullptr || hidden_ref != nullptr;
+  if (!w1) w1 = w0;
+  if (!hidden_ref) hidden_ref = hidden;
   char* ws = static_cast<char*>(workspace);
   const FusedPlan plan = fused_plan(n_tokens, H, V);
   int32_t* n_valid = nullptr;
@@ -1061,11 +1066,20 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, floa
   a.hidden_stride_b = (uint32_t)(hidden_stride * 2);
   a.weight_stride_b = (uint32_t)(weight_stride * 2);
   a.hidden_bytes = (uint32_t)(((n_tokens - 1) * hidden_stride + H) * 2);
+  const char* second_hidden = static_cast<const char*>(hidden_ref);
   if (norm_weight) {  // normalise the valid rows into a dense buffer and multiply that
-    char* normed = ws + off_partials(n_tokens) + (w1 ? 2 : 1) * partial_bytes(n_tokens, H, V);
+    char* normed = ws + off_partials(n_tokens) + (second ? 2 : 1) * partial_bytes(n_tokens, H, V);
     NormArgs na{a.hidden, static_cast<const uint16_t*>(norm_weight), normed, row_index, n_valid,
                 a.hidden_stride_b, (int)n_tokens, (int)H, norm_eps};
     hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, stream, na);
+    if (hidden_ref != hidden) {
+      na.x = static_cast<const char*>(hidden_ref);
+      na.y = normed + normed_bytes(n_tokens, H, true);
+      hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, stream, na);
+      second_hidden = na.y;
+    } else {
+      second_hidden = normed;
+    }
     a.hidden = normed;
     a.hidden_index = nullptr;
     a.hidden_stride_b = (uint32_t)(H * 2);
@@ -1087,17 +1101,20 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, floa
   a.partials = p0;
   if (out_entropy) launch_main<true>(a, plan.kind, plan.grid, out_argmax != nullptr, stream);
   else launch_main<false>(a, plan.kind, plan.grid, out_argmax != nullptr, stream);
-  if (w1) {
+  const char* first_hidden = a.hidden;
+  if (second) {
     a.weight = static_cast<const char*>(w1);
+    a.hidden = second_hidden;
     a.partials = p1;
     launch_main<false>(a, plan.kind, plan.grid, false, stream);
+    a.hidden = first_hidden;
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
 
   CombineArgs c;
   c.partials = p0;
-  c.partials_ref = w1 ? p1 : nullptr;
+  c.partials_ref = second ? p1 : nullptr;
   c.row_index = row_index;
   c.n_valid = n_valid;
   c.out_lp = out_lp;
@@ -1119,6 +1136,27 @@ hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, floa
   c.scale = a.scale;
   hipLaunchKernelGGL(fused_combine_kernel, dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, stream, c);
   return hipGetLastError();
+}
+
+hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, float norm_eps, const void* w0,
+                               const void* w1, int64_t n_tokens, int64_t H, int64_t V, int64_t hidden_stride,
+                               int64_t weight_stride, const int32_t* targets,
+                               const int32_t* row_valid, float temperature, float* out_lp, float* out_lse,
+                               float* out_entropy, int32_t* out_argmax, float* out_ref_lp, float* out_k3,
+                               void* workspace, hipStream_t stream) {
+  return fused_launch_impl(hidden, nullptr, norm_weight, norm_eps, w0, w1, n_tokens, H, V, hidden_stride, weight_stride,
+                           targets, row_valid, temperature, out_lp, out_lse, out_entropy, out_argmax, out_ref_lp, out_k3,
+                           workspace, stream);
+}
+
+hipError_t fused_pair_launch(const void* hidden, const void* hidden_ref, const void* norm_weight, float norm_eps,
+                             const void* w0, const void* w1, int64_t n_tokens, int64_t H, int64_t V,
+                             int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
+                             const int32_t* row_valid, float temperature, float* out_lp, float* out_entropy,
+                             float* out_ref_lp, float* out_k3, void* workspace, hipStream_t stream) {
+  return fused_launch_impl(hidden, hidden_ref, norm_weight, norm_eps, w0, w1, n_tokens, H, V, hidden_stride,
+                           weight_stride, targets, row_valid, temperature, out_lp, nullptr, out_entropy, nullptr,
+                           out_ref_lp, out_k3, workspace, stream);
 }
 
 }  // namespace tome

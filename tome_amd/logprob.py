@@ -393,3 +393,49 @@ def grpo_dual_logprobs(hidden: torch.Tensor, w_policy: torch.Tensor, w_ref: torc
                                       temperature, outs[0].data_ptr(), outs[1].data_ptr(), outs[2].data_ptr(),
                                       outs[3].data_ptr(), _ptr(ws), ws_bytes, _stream(dev)))
     return DualLogprobs(*(o.reshape(lead) for o in outs))
+
+
+def grpo_pair_logprobs(hidden_policy: torch.Tensor, hidden_ref: torch.Tensor, w_policy: torch.Tensor, targets,
+                       temperature: float = 1.0, lengths=None, *, w_ref: torch.Tensor | None = None,
+                       row_valid=None, norm_weight: torch.Tensor | None = None,
+                       norm_eps: float = 1e-6) -> DualLogprobs:
+    """``grpo_dual_logprobs`` for the reference's two-model layout: one hidden-state matrix per model.
+
+    Tome's ``UpdateWeights`` merges LoRA deltas into attention and MLP weights only
+    (mlx-impl/node.py:134-151), so policy and reference models differ in their final hidden
+    states and share the final norm and the lm_head (mlx-impl/model.py:536-538): ``w_ref``
+    defaults to ``w_policy``.  ``norm_weight`` as in ``fused_lmhead_logprobs``, applied to both.
+    """
+    lib = _lib.load_library()
+    ws_in = (w_policy,) if w_ref is None else (w_policy, w_ref)
+    dev, lead, h2, ws_ = _check_fused_inputs(hidden_policy, *ws_in)
+    _require_gpu(hidden_policy, hidden_ref)
+    if hidden_ref.dtype != torch.bfloat16 or hidden_ref.shape != hidden_policy.shape:
+        raise ValueError("hidden_ref must be bfloat16 with hidden_policy's shape")
+    r2 = _rows_view(hidden_ref)
+    wp = ws_[0]
+    wr = ws_[1] if w_ref is not None else wp
+    if wp.stride(0) != wr.stride(0):
+        wp, wr = wp.contiguous(), wr.contiguous()
+    n, H = h2.shape
+    if n > 1 and h2.stride(0) != r2.stride(0):
+        h2, r2 = h2.contiguous(), r2.contiguous()
+    temperature = _check_temperature(temperature)
+    V = wp.shape[0]
+    tg = _as_i32(targets, n, dev, "targets")
+    rv = _row_valid(lead, n, lengths, row_valid, dev)
+    nw = None
+    if norm_weight is not None:
+        _require_gpu(hidden_policy, norm_weight)
+        if norm_weight.dtype != torch.bfloat16 or norm_weight.shape != (H,):
+            raise ValueError(f"norm_weight must be bfloat16 [{H}]")
+        nw = norm_weight.contiguous()
+    with _on_device(dev):
+        outs = [torch.empty(n, dtype=torch.float32, device=dev) for _ in range(4)]
+        ws_bytes = lib.tome_grpo_pair_workspace(n, H, V, 1 if nw is not None else 0)
+        ws = _workspace(ws_bytes, dev)
+        _lib.check(lib.tome_grpo_pair(h2.data_ptr(), r2.data_ptr(), _ptr(nw), float(norm_eps), wp.data_ptr(),
+                                      wr.data_ptr(), n, H, V, h2.stride(0) if n > 1 else H, wp.stride(0),
+                                      tg.data_ptr(), _ptr(rv), temperature, outs[0].data_ptr(), outs[1].data_ptr(),
+                                      outs[2].data_ptr(), outs[3].data_ptr(), _ptr(ws), ws_bytes, _stream(dev)))
+    return DualLogprobs(*(o.reshape(lead) for o in outs))
