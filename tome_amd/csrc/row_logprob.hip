@@ -50,18 +50,23 @@ __device__ __forceinline__ int argmax_in_unit(const T* row, int64_t V, int unit,
   return (int)first;
 }
 
+// The target's logit, or NaN when no log-prob is asked for or the id is outside [0, V).  Lane 0 issues
+// this at the start of its workgroup, so the dependent load pair (id, then logit) is long finished
+// when the row has been streamed.
+template <typename T>
+__device__ __forceinline__ float load_target_logit(const RowArgs& a, const T* row, int64_t r) {
+  if (!a.out_lp || !a.targets) return __builtin_nanf("");
+  const int32_t t = a.targets[r];
+  return (t >= 0 && t < a.V) ? Elem<T>::load1(row + t) : __builtin_nanf("");
+}
+
 template <typename T, bool ENT, bool AMAX>
-__device__ __forceinline__ void finish_row(const RowArgs& a, const T* row, int64_t r, const RowStat& st) {
+__device__ __forceinline__ void finish_row(const RowArgs& a, const T* row, int64_t r, const RowStat& st, float x_t) {
   // Called by one lane.  lp = (y_t - m - log2 s) ln2 with the same fma that fed the sum, so
   // the target's own term is part of s and lp <= 0 up to the rounding of the merges.
   const float m = st.mx * a.scale;
   const float log2s = fast_log2(st.s);
-  const int32_t t = a.targets ? a.targets[r] : -1;
-  if (a.out_lp) {
-    float lp = __builtin_nanf("");
-    if (t >= 0 && t < a.V) lp = (fmaf(Elem<T>::load1(row + t), a.scale, -m) - log2s) * kLn2;
-    a.out_lp[r] = lp;
-  }
+  if (a.out_lp) a.out_lp[r] = (fmaf(x_t, a.scale, -m) - log2s) * kLn2;  // NaN in, NaN out
   if (a.out_lse) a.out_lse[r] = (m + log2s) * kLn2;
   if constexpr (ENT) a.out_entropy[r] = (m + log2s - st.w / st.s) * kLn2;
   if constexpr (AMAX) a.out_argmax[r] = argmax_in_unit<T, true>(row, a.V, st.bi, st.mx);
@@ -91,6 +96,8 @@ __global__ __launch_bounds__(kRowWG) void row_logprob_kernel(RowArgs a) {
   const int64_t u0 = per_split * split;
   const int64_t u1 = (u0 + per_split < n_units) ? u0 + per_split : n_units;
 
+  float x_t = 0.f;
+  if (tid == 0 && a.splits == 1) x_t = load_target_logit<T>(a, row, r);
   RowStat st = stat_identity();
   if constexpr (VECTOR) {
     const u32x4* p = reinterpret_cast<const u32x4*>(row);
@@ -137,12 +144,12 @@ __global__ __launch_bounds__(kRowWG) void row_logprob_kernel(RowArgs a) {
   if (tid != 0) return;
   if (a.splits == 1) {
     if constexpr (VECTOR) {
-      finish_row<T, ENT, AMAX>(a, row, r, tot);
+      finish_row<T, ENT, AMAX>(a, row, r, tot, x_t);
     } else {
       // Scalar path: unit index == element index.
       RowArgs b = a;
       b.out_argmax = nullptr;
-      finish_row<T, ENT, false>(b, row, r, tot);
+      finish_row<T, ENT, false>(b, row, r, tot, x_t);
       if constexpr (AMAX) a.out_argmax[r] = tot.bi < a.V ? tot.bi : 0;
     }
   } else {
@@ -156,6 +163,9 @@ __global__ __launch_bounds__(64) void row_combine_kernel(RowArgs a) {
   const int64_t r = blockIdx.x;
   if (a.row_valid && a.row_valid[r] == 0) return;  // outputs already zeroed by the main kernel
   const int lane = threadIdx.x;
+  const T* row = static_cast<const T*>(a.logits) + r * a.row_stride;
+  float x_t = 0.f;
+  if (lane == 0) x_t = load_target_logit<T>(a, row, r);
   RowStat st = stat_identity();
   if (lane < a.splits) {
     const RowPartial p = a.partials[r * a.splits + lane];
@@ -163,13 +173,12 @@ __global__ __launch_bounds__(64) void row_combine_kernel(RowArgs a) {
   }
   stat_wave_reduce(st, a.scale);
   if (lane != 0) return;
-  const T* row = static_cast<const T*>(a.logits) + r * a.row_stride;
   if constexpr (VECTOR) {
-    finish_row<T, ENT, AMAX>(a, row, r, st);
+    finish_row<T, ENT, AMAX>(a, row, r, st, x_t);
   } else {
     RowArgs b = a;
     b.out_argmax = nullptr;
-    finish_row<T, ENT, false>(b, row, r, st);
+    finish_row<T, ENT, false>(b, row, r, st, x_t);
     if constexpr (AMAX) a.out_argmax[r] = st.bi < a.V ? st.bi : 0;
   }
 }
