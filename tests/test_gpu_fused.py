@@ -262,3 +262,29 @@ def test_norm_lmhead_matches_oracle(dev, n, H, V, masked):
     # the norm must really have been applied: without it the answer is far away
     raw = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 0.9).lp.cpu().numpy()
     assert np.abs(raw[m] - want["lp"][m]).max() > 0.1
+
+
+@pytest.mark.parametrize("n,H,V,masked", [
+    (1, 1024, 151936, False), (16, 1024, 40000, True), (17, 1024, 8191, False), (64, 1024, 151936, True),
+    (33, 2048, 30001, False), (64, 2048, 12345, True), (9, 4096, 20000, False), (32, 4096, 33000, True),
+    (20, 2560, 9000, False), (5, 512, 7000, False), (64, 1536, 5000, False), (48, 1024, 70, False)])
+def test_fused_small_batch_kernel(dev, n, H, V, masked):
+    """Decode-sized batches (<= 64 tokens) take the streaming kernel with K split across waves (where the shape
+    rules allow it; the other shapes here fall back to the tiled kernel) - same bar either way."""
+    rng = np.random.default_rng(n * 31 + H + V)
+    h, w, t = _inputs(dev, n, H, V, n * 31 + H + V, w_scale=0.05)
+    valid = (rng.random(n) < 0.7).astype(np.int32) if masked else np.ones(n, dtype=np.int32)
+    if masked:
+        valid[rng.integers(0, n)] = 1
+    r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 0.8, want_lse=True, want_entropy=True,
+                                       want_argmax=True, row_valid=torch.from_numpy(valid).to(dev) if masked else None)
+    want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(w), t, 0.8)
+    m = valid.astype(bool)
+    np.testing.assert_allclose(r.lp.cpu().numpy()[m], want["lp"][m], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.lse.cpu().numpy()[m], want["lse"][m], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.entropy.cpu().numpy()[m], want["entropy"][m], atol=TOL, rtol=0)
+    clear = m & ((want["top1"] - want["top2"]) > 1e-2)
+    np.testing.assert_array_equal(r.argmax.cpu().numpy()[clear], want["argmax"][clear])
+    assert (r.lp.cpu().numpy()[~m] == 0).all() and (r.argmax.cpu().numpy()[~m] == -1).all()
+    plain = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 0.8)     # the variant without extras
+    np.testing.assert_allclose(plain.lp.cpu().numpy(), want["lp"], atol=TOL, rtol=0)

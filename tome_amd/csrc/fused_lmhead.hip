@@ -15,7 +15,9 @@
 //     that share a token are merged once at the end.
 //   * A workgroup owns one token tile and a contiguous range of 256-row vocab tiles.  Per vocab
 //     tile it runs the K loop, then folds the accumulator tile into the running
-//     (max, sum 2^(y-m), sum y 2^(y-m)) states.  Two kernels share this shape:
+//     (max, sum 2^(y-m), sum y 2^(y-m)) states.  Two kernels share this shape; a third,
+//     fused_lmhead_small_kernel (<= 64 tokens, W streamed once, K split across waves), is
+//     described where it is defined:
 //       fused_lmhead_dma_kernel  (H % 64 == 0, more than 128 tokens) 512 lanes, 256 x 256 tile,
 //                                16x16x32 MFMA, K slabs DMA'd into LDS - described at the kernel;
 //       fused_lmhead_kernel      (any H % 8, short batches) 256 lanes, 256 x 128 tile, 32x32x16
@@ -728,6 +730,108 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
                    sch.n_splits * kPartsPerSplit, l16, g, a.scale);
 }
 
+// ===============================================================================================
+// Small batches (<= 64 tokens, the decode-step regime): W streams from HBM exactly once and nothing is
+// reused, so the kernel is built like a streaming reduction, not like a GEMM.
+//
+//   * K is split across the waves of a workgroup (256 or 512 columns each).  A wave's slice of the
+//     hidden states - all tokens - then fits its registers as MFMA B fragments for the whole launch,
+//     and W goes from global memory straight into A fragments: no LDS staging, no barrier on the
+//     load path.
+//   * Each wave keeps 16 sixteen-byte loads in flight (two 16-row tiles of its K slice, refilled in
+//     place right after the MFMA that consumed them); one workgroup per CU owns one contiguous range of
+//     16-row vocab tiles.
+//   * Per tile the waves' partial sums (16 rows x 16*NBT tokens, MFMA layout) meet in LDS; wave j sums
+//     them in wave order and folds token block j into its online-softmax state.  One barrier per tile:
+//     the buffer of tile t is rewritten at tile t + 2, after the barrier of tile t + 1, which the
+//     folding waves only reach once tile t is folded.
+//   * One partial per (token, workgroup); the combine kernel is shared with the other paths.
+// ===============================================================================================
+template <bool ENT, bool AMAX, int NBT, int KSTEPS>
+__global__ __launch_bounds__(512) void fused_lmhead_small_kernel(FusedArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char small_mem[];  // [2][waves][NBT][64 lanes] f32x4
+  constexpr int kBuf = 16 / KSTEPS;                                 // tile buffers in flight: 2 or 1
+  const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
+  if (n_valid <= 0) return;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n_waves = blockDim.x >> 6;
+  const int l16 = lane & 15, g = lane >> 4;
+  const int n_tiles = (a.V + 15) >> 4;
+  const int t0 = (int)((int64_t)blockIdx.x * n_tiles / gridDim.x);
+  const int t1 = (int)((int64_t)(blockIdx.x + 1) * n_tiles / gridDim.x);
+  const int kb0 = (wave * KSTEPS * 32 + 8 * g) * 2;  // byte offset of this lane's first K chunk in a row
+
+  // Hidden-state fragments of this wave's K slice: lane (token l16, group g) holds K = 32 ks + 8 g .. + 7.
+  bf16x8 fb[KSTEPS][NBT];
+#pragma unroll
+  for (int j = 0; j < NBT; ++j) {
+    int p = j * 16 + l16;
+    p = p < n_valid ? p : n_valid - 1;
+    const int tok = a.hidden_index ? a.hidden_index[p] : p;
+    const char* hp = a.hidden + (int64_t)tok * a.hidden_stride_b + kb0;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) fb[ks][j] = *reinterpret_cast<const bf16x8*>(hp + ks * 64);
+  }
+  // Token state of the block this wave folds (waves >= NBT fold nothing).
+  RowStat st[1] = {stat_identity()};
+  float tx[1] = {-INFINITY};
+  int tgt[1] = {-1};
+  if (wave < NBT) {
+    const int p = wave * 16 + l16;
+    int t = -1;
+    if (p < n_valid) t = a.targets[a.row_index ? a.row_index[p] : p];
+    tgt[0] = (t >= 0 && t < a.V) ? t : -1;
+  }
+
+  auto w_ptr = [&](int t) {  // rows past V (last tile only) read the last row; masked in the fold
+    int row = t * 16 + l16;
+    row = row < a.V ? row : a.V - 1;
+    return a.weight + (int64_t)row * a.weight_stride_b + kb0;
+  };
+  u32x4 wb[kBuf][KSTEPS];
+#pragma unroll
+  for (int b = 0; b < kBuf && t0 < t1; ++b) {
+    const char* wp = w_ptr(t0 + b < t1 ? t0 + b : t1 - 1);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) wb[b][ks] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + ks * 64));
+  }
+
+  for (int tb = t0; tb < t1; tb += kBuf) {
+#pragma unroll
+    for (int b = 0; b < kBuf; ++b) {
+      const int t = tb + b;
+      if (t >= t1) break;  // uniform
+      // The refill is unconditional (past the range it re-reads the tile just consumed, an L2 hit that is
+      // never used): with a load behind a branch the compiler cannot count the loads in flight and waits
+      // for far more of them than the one it needs.
+      const char* wnext = w_ptr(t + kBuf < t1 ? t + kBuf : t);
+      f32x4v acc[NBT];
+#pragma unroll
+      for (int j = 0; j < NBT; ++j) acc[j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const bf16x8 fa = __builtin_bit_cast(bf16x8, wb[b][ks]);
+#pragma unroll
+        for (int j = 0; j < NBT; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, fb[ks][j], acc[j], 0, 0, 0);
+        wb[b][ks] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wnext + ks * 64));
+      }
+      char* red = small_mem + (size_t)(((t & 1) * n_waves + wave) * NBT) * 1024 + lane * 16;
+#pragma unroll
+      for (int j = 0; j < NBT; ++j) *reinterpret_cast<f32x4v*>(red + j * 1024) = acc[j];
+      __syncthreads();
+      if (wave < NBT) {
+        f32x4v sum[1][1] = {{f32x4v{0.f, 0.f, 0.f, 0.f}}};
+        const char* src = small_mem + (size_t)((t & 1) * n_waves * NBT + wave) * 1024 + lane * 16;
+        for (int w = 0; w < n_waves; ++w) sum[0][0] += *reinterpret_cast<const f32x4v*>(src + (size_t)w * NBT * 1024);
+        fold_tile16<ENT, AMAX, 1, 1>(sum, st, tx, tgt, t * 16, g, t * 16 + 16 > a.V, a.V, a.scale);
+      }
+    }
+  }
+  // One partial per (token, workgroup): part index = workgroup id.
+  if (wave < NBT) write_partials16<1>(st, tx, a.partials, wave * 16, n_valid, (int)blockIdx.x, (int)gridDim.x, l16, g, a.scale);
+}
+
 // ---- compaction of valid rows ----------------------------------------------------------------
 // One workgroup: row_index[0 .. n_valid) = ascending indices of rows with row_valid != 0.
 // Outputs of masked rows are zeroed here.
@@ -954,22 +1058,75 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
 // The DMA kernel needs whole 64-wide K slabs and pays for 256-token tiles; short batches and ragged H
 // go to the generic kernel.
 
-enum FusedKind { kGeneric = 0, kDma = 1 };
+enum FusedKind { kGeneric = 0, kDma = 1, kSmall = 2 };
 
 struct FusedPlan {
   FusedKind kind;
+  int small_nbt, small_ksteps, small_waves;  // kSmall only
   int bt, bv, slots, n_vtiles;
   int grid;            // workgroups to launch: the most any number of valid tokens can ask for
   size_t max_records;  // partial records any number of valid tokens can produce
 };
 
+template <typename K>
+static void allow_big_lds(K kernel, int bytes) {
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+// Workgroups of the small-batch kernel: one per CU.  Measured at 16 and 64 tokens, H = 1024: 256 workgroups
+// 59 us, 512 66 us, 1024 (all that fit) 71 us, 2048 (queued) 95 us; a deeper load ring changes nothing.
+// The stream is bound by the 16-rows-by-64-bytes shape of an MFMA operand load, which a plain copy
+// kernel of the same shape and lifetime moves at 5.6 TB/s, and more concurrent streams lower that.
+static int small_wg_count() {
+  static int n = 0;
+  if (n == 0) {
+    int cus = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 2)
+      return 0;
+    if (cus > 512) cus = 512;  // the workspace holds 512 parts per token
+    n = cus & ~1;              // even: the combine kernel counts parts in pairs
+  }
+  return n;
+}
+
+// Shape rules of the small-batch kernel: <= 64 tokens, K split over 2..8 waves in slices of 256 or 512.
+static bool small_shape(int64_t n_tokens, int64_t H, int64_t V, int& nbt, int& ksteps, int& waves) {
+  if (n_tokens > 64 || V < 64) return false;
+  nbt = n_tokens <= 16 ? 1 : (n_tokens <= 32 ? 2 : 4);
+  if (H % 256 == 0 && H / 256 <= 8 && H / 256 >= 2) {
+    ksteps = 8;
+    waves = (int)(H / 256);
+  } else if (H % 512 == 0 && H / 512 <= 8 && H / 512 >= 2 && nbt <= 2) {
+    ksteps = 16;
+    waves = (int)(H / 512);
+  } else {
+    return false;
+  }
+  if (ksteps == 8 && nbt == 2) nbt = 4;  // instantiated token-block counts: 1 and 4 (K 256), 1 and 2 (K 512)
+  return waves >= nbt;
+}
+
 static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   FusedPlan p;
   p.kind = kGeneric;
+  p.small_nbt = p.small_ksteps = p.small_waves = 0;
   if (n_tokens > kBT && H % k2BK == 0) p.kind = kDma;
+  if (small_shape(n_tokens, H, V, p.small_nbt, p.small_ksteps, p.small_waves)) p.kind = kSmall;
   if (const char* ov = getenv("TOME_FUSED_KERNEL")) {  // tuning knob: force a path where its shape rules allow
     if (ov[0] == 'g') p.kind = kGeneric;
     if (ov[0] == 'd' && H % k2BK == 0) p.kind = kDma;
+  }
+  p.n_vtiles = 0;
+  if (p.kind == kSmall) {
+    // One partial per (token, workgroup); one workgroup per CU, at most 512.
+    p.bt = 64;
+    p.bv = 16;
+    p.slots = 1;     // only feed the schedule that the compaction kernel writes and this path ignores
+    p.n_vtiles = 1;
+    p.grid = 0;
+    p.max_records = (size_t)64 * 512;
+    return p;
   }
   p.bt = p.kind == kGeneric ? kBT : k2BT;   // the DMA path has a 256 x 256 tile
   p.bv = p.kind == kGeneric ? kBV : k2BV;
@@ -1003,11 +1160,6 @@ size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weigh
   return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, H, V) + normed_bytes(n_tokens, H, with_norm);
 }
 
-template <typename K>
-static void allow_big_lds(K kernel, int bytes) {
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-}
-
 template <bool ENT, bool AMAX>
 static void launch_dma(const FusedArgs& a, int grid, hipStream_t stream) {
   static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
@@ -1018,14 +1170,41 @@ static void launch_dma(const FusedArgs& a, int grid, hipStream_t stream) {
   hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX>), dim3((unsigned)grid), dim3(k2WG), k2LdsTotal, stream, a);
 }
 
+template <bool ENT, bool AMAX, int NBT, int KSTEPS>
+static int launch_small(const FusedArgs& a, int waves, hipStream_t stream) {
+  int n_wg = small_wg_count();
+  const int n_tiles = (a.V + 15) / 16;
+  if (n_wg > n_tiles) n_wg = n_tiles & ~1;  // no empty vocab ranges
+  if (n_wg < 2) return 0;
+  const size_t lds = (size_t)2 * waves * NBT * 1024;
+  hipLaunchKernelGGL((fused_lmhead_small_kernel<ENT, AMAX, NBT, KSTEPS>), dim3((unsigned)n_wg), dim3((unsigned)waves * 64),
+                     lds, stream, a);
+  return n_wg;
+}
+
+// Launches the sweep kernel of `plan`.  Returns the number of partials per token it leaves (0 = the
+// schedule's own count), or -1 when the small-batch kernel could not be placed.
 template <bool ENT>
-static void launch_main(const FusedArgs& a, FusedKind kind, int grid, bool want_argmax, hipStream_t stream) {
-  if (kind == kDma) {
-    if (want_argmax) launch_dma<ENT, true>(a, grid, stream);
-    else launch_dma<ENT, false>(a, grid, stream);
-  } else {
-    hipLaunchKernelGGL(fused_lmhead_kernel<ENT>, dim3((unsigned)grid), dim3(kFusedWG), 0, stream, a);
+static int launch_main(const FusedArgs& a, const FusedPlan& plan, bool want_argmax, hipStream_t stream) {
+  if (plan.kind == kSmall) {
+    int n = 0;
+    const int w = plan.small_waves;
+#define TOME_SMALL(NBT, KS)                                                 \
+  n = want_argmax ? launch_small<ENT, true, NBT, KS>(a, w, stream) : launch_small<ENT, false, NBT, KS>(a, w, stream)
+    if (plan.small_ksteps == 8 && plan.small_nbt == 1) TOME_SMALL(1, 8);
+    else if (plan.small_ksteps == 8) TOME_SMALL(4, 8);
+    else if (plan.small_nbt == 1) TOME_SMALL(1, 16);
+    else TOME_SMALL(2, 16);
+#undef TOME_SMALL
+    return n >= 2 ? n : -1;
   }
+  if (plan.kind == kDma) {
+    if (want_argmax) launch_dma<ENT, true>(a, plan.grid, stream);
+    else launch_dma<ENT, false>(a, plan.grid, stream);
+  } else {
+    hipLaunchKernelGGL(fused_lmhead_kernel<ENT>, dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
+  }
+  return 0;
 }
 
 // One sweep per (hidden, weight) pair: the policy pair always, and a reference pair when a second weight
@@ -1099,14 +1278,19 @@ static hipError_t fused_launch_impl(const void* hidden, const void* hidden_ref, 
 
   a.weight = static_cast<const char*>(w0);
   a.partials = p0;
-  if (out_entropy) launch_main<true>(a, plan.kind, plan.grid, out_argmax != nullptr, stream);
-  else launch_main<false>(a, plan.kind, plan.grid, out_argmax != nullptr, stream);
+  int n_parts = out_entropy ? launch_main<true>(a, plan, out_argmax != nullptr, stream)
+                            : launch_main<false>(a, plan, out_argmax != nullptr, stream);
+  if (n_parts < 0) return hipErrorLaunchFailure;
+  if (n_parts > 0) {  // small-batch kernel: one part per workgroup, whatever the mask
+    a.sched = FusedSchedule{1, n_parts / kPartsPerSplit, n_parts, 0};
+    a.sched_dev = nullptr;
+  }
   const char* first_hidden = a.hidden;
   if (second) {
     a.weight = static_cast<const char*>(w1);
     a.hidden = second_hidden;
     a.partials = p1;
-    launch_main<false>(a, plan.kind, plan.grid, false, stream);
+    if (launch_main<false>(a, plan, false, stream) < 0) return hipErrorLaunchFailure;
     a.hidden = first_hidden;
   }
   hipError_t e = hipGetLastError();
