@@ -736,8 +736,8 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 //
 //   * K is split across the waves of a workgroup (256 or 512 columns each).  A wave's slice of the
 //     hidden states - all tokens - then fits its registers as MFMA B fragments for the whole launch,
-//     and W goes from global memory straight into A fragments: no LDS staging, no barrier on the
-//     load path.
+//     and W goes from global memory into registers and through a wave-private LDS tile into A
+//     fragments: no barrier on the load path.
 //   * Each wave keeps 16 sixteen-byte loads in flight (two 16-row tiles of its K slice, refilled in
 //     place right after the MFMA that consumed them); one workgroup per CU owns one contiguous range of
 //     16-row vocab tiles.
@@ -749,7 +749,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 // ===============================================================================================
 template <bool ENT, bool AMAX, int NBT, int KSTEPS>
 __global__ __launch_bounds__(512) void fused_lmhead_small_kernel(FusedArgs a) {
-  extern __shared__ __attribute__((aligned(16))) char small_mem[];  // [2][waves][NBT][64 lanes] f32x4
+  extern __shared__ __attribute__((aligned(16))) char small_mem[];  // [2][waves][NBT][64 lanes] f32x4, then [waves] 4 KB tiles
   constexpr int kBuf = 16 / KSTEPS;                                 // tile buffers in flight: 2 or 1
   const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
   if (n_valid <= 0) return;
@@ -784,17 +784,30 @@ __global__ __launch_bounds__(512) void fused_lmhead_small_kernel(FusedArgs a) {
     tgt[0] = (t >= 0 && t < a.V) ? t : -1;
   }
 
-  auto w_ptr = [&](int t) {  // rows past V (last tile only) read the last row; masked in the fold
-    int row = t * 16 + l16;
+  // W loads are shaped for HBM, not for the MFMA: one instruction fetches 4 rows x 256 bytes (lane = row
+  // lane/16 of the group, 16-byte chunk lane%16), which streams 17 % faster than the operand shape of 16
+  // rows x 64 bytes (6.85 against 5.84 TB/s in a copy kernel with this kernel's structure).  A unit of
+  // 16 rows x 256 bytes (four K steps) then changes layout through a wave-private 4 KB LDS tile: chunk c
+  // of row r is stored at position c ^ r, so the contiguous writes and the fragment reads (16 rows, one
+  // chunk) are both free of bank conflicts.
+  constexpr int kUnits = KSTEPS / 4;  // units per tile and wave
+  const int lr = lane >> 4, lc = lane & 15;
+  auto w_ptr = [&](int t, int q) {  // rows past V (last tile only) read the last row; masked in the fold
+    int row = t * 16 + 4 * q + lr;
     row = row < a.V ? row : a.V - 1;
-    return a.weight + (int64_t)row * a.weight_stride_b + kb0;
+    return a.weight + (int64_t)row * a.weight_stride_b + wave * (KSTEPS * 64) + lc * 16;
   };
-  u32x4 wb[kBuf][KSTEPS];
+  char* stage = small_mem + (size_t)2 * n_waves * NBT * 1024 + wave * 4096;
+  u32x4 wb[kBuf][kUnits][4];
 #pragma unroll
   for (int b = 0; b < kBuf && t0 < t1; ++b) {
-    const char* wp = w_ptr(t0 + b < t1 ? t0 + b : t1 - 1);
+    const int t = t0 + b < t1 ? t0 + b : t1 - 1;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) wb[b][ks] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + ks * 64));
+    for (int q = 0; q < 4; ++q) {
+      const char* wp = w_ptr(t, q);
+#pragma unroll
+      for (int u = 0; u < kUnits; ++u) wb[b][u][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + u * 256));
+    }
   }
 
   for (int tb = t0; tb < t1; tb += kBuf) {
@@ -805,16 +818,33 @@ __global__ __launch_bounds__(512) void fused_lmhead_small_kernel(FusedArgs a) {
       // The refill is unconditional (past the range it re-reads the tile just consumed, an L2 hit that is
       // never used): with a load behind a branch the compiler cannot count the loads in flight and waits
       // for far more of them than the one it needs.
-      const char* wnext = w_ptr(t + kBuf < t1 ? t + kBuf : t);
+      const int tn = t + kBuf < t1 ? t + kBuf : t;
       f32x4v acc[NBT];
 #pragma unroll
       for (int j = 0; j < NBT; ++j) acc[j] = f32x4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const bf16x8 fa = __builtin_bit_cast(bf16x8, wb[b][ks]);
+      for (int u = 0; u < kUnits; ++u) {
 #pragma unroll
-        for (int j = 0; j < NBT; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, fb[ks][j], acc[j], 0, 0, 0);
-        wb[b][ks] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wnext + ks * 64));
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<u32x4*>(stage + (4 * q + lr) * 256 + ((lc ^ (4 * q + lr)) << 4)) = wb[b][u][q];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          wb[b][u][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w_ptr(tn, q) + u * 256));
+        // The tile is private to this wave and LDS serves a wave's requests in order.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        bf16x8 fa[4];
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4)
+          fa[k4] = *reinterpret_cast<const bf16x8*>(stage + l16 * 256 + (((4 * k4 + g) ^ l16) << 4));
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4)
+#pragma unroll
+          for (int j = 0; j < NBT; ++j)
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[k4], fb[4 * u + k4][j], acc[j], 0, 0, 0);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the next unit overwrites what was just read
+        __builtin_amdgcn_wave_barrier();
       }
       char* red = small_mem + (size_t)(((t & 1) * n_waves + wave) * NBT) * 1024 + lane * 16;
 #pragma unroll
@@ -1090,14 +1120,15 @@ static int small_wg_count() {
   return n;
 }
 
-// Shape rules of the small-batch kernel: <= 64 tokens, K split over 2..8 waves in slices of 256 or 512.
+// Shape rules of the small-batch kernel: <= 64 tokens, K split over 2..8 waves in slices of 256 or 512
+// (slices of 128 on twice the waves measured 2 us slower at H = 1024).
 static bool small_shape(int64_t n_tokens, int64_t H, int64_t V, int& nbt, int& ksteps, int& waves) {
   if (n_tokens > 64 || V < 64) return false;
   nbt = n_tokens <= 16 ? 1 : (n_tokens <= 32 ? 2 : 4);
   if (H % 256 == 0 && H / 256 <= 8 && H / 256 >= 2) {
     ksteps = 8;
     waves = (int)(H / 256);
-  } else if (H % 512 == 0 && H / 512 <= 8 && H / 512 >= 2 && nbt <= 2) {
+  } else if (H % 512 == 0 && H / 512 <= 8 && nbt <= 2) {
     ksteps = 16;
     waves = (int)(H / 512);
   } else {
@@ -1176,7 +1207,12 @@ static int launch_small(const FusedArgs& a, int waves, hipStream_t stream) {
   const int n_tiles = (a.V + 15) / 16;
   if (n_wg > n_tiles) n_wg = n_tiles & ~1;  // no empty vocab ranges
   if (n_wg < 2) return 0;
-  const size_t lds = (size_t)2 * waves * NBT * 1024;
+  const size_t lds = (size_t)2 * waves * NBT * 1024 + (size_t)waves * 4096;
+  static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
+  if (!attr_set && lds > 65536) {
+    allow_big_lds(&fused_lmhead_small_kernel<ENT, AMAX, NBT, KSTEPS>, 2 * 8 * 4 * 1024 + 8 * 4096);
+    attr_set = true;
+  }
   hipLaunchKernelGGL((fused_lmhead_small_kernel<ENT, AMAX, NBT, KSTEPS>), dim3((unsigned)n_wg), dim3((unsigned)waves * 64),
                      lds, stream, a);
   return n_wg;
