@@ -32,6 +32,7 @@ TRAFFIC_ROW_MASKED = 716.6e6 + 0.13e6
 TRAFFIC_ROW_ALL = 1245.4e6 + 0.13e6
 TRAFFIC_FUSED_CFG3 = 1826e6 + 6.8e6
 TRAFFIC_DECODE_64 = 39.4e6 + 0.42e6 + 0.40e6   # sampler: main-kernel fetch, combine fetch, partials written
+TRAFFIC_FUSED_SMALL_64 = 326.0e6 + 0.52e6      # sweep kernel: fetch + partials written (profiles/fused_lmhead_small_kernel_decode_64tokens.txt)
 TRAFFIC_LORA_06B = 812.1e6 + 763.4e6            # merge kernel: fetch + write (profiles/lora_merge_kernel_qwen3_0.6b_update.txt)
 
 
@@ -121,12 +122,13 @@ def bench_row(dev, steps, warmup, variant="both"):
     return out
 
 
-def bench_fused(dev, steps, warmup):
+def bench_fused(dev, steps, warmup, n=4096, H=1024):
+    """Fused lm_head + log-softmax on [n, H] x [V, H]: config 3 by default; n = 64 is the decode-step batch,
+    where W is streamed once and the kernel is HBM-bound."""
     import torch
     import tome_amd
     from tome_amd import _lib
     lib = tome_amd.load_library()
-    n, H = 4096, 1024
     g = torch.Generator(device=dev).manual_seed(4321)
     hidden = torch.randn((n, H), device=dev, generator=g).to(torch.bfloat16)
     weight = (torch.randn((V, H), device=dev, generator=g) * 0.02).to(torch.bfloat16)
@@ -219,7 +221,7 @@ def bench_lora(dev, steps, warmup):
     return {"ms": ms, "wall_ms": wall, "bytes": n_bytes, "jobs": len(jobs), "rank": rank}
 
 
-def cpu_baseline(sample_rows=256, budget_s=12.0):
+def cpu_baseline(sample_rows=1024, budget_s=12.0):
     """NumPy fp32 restatement of local_compute_logprobs (mlx-impl/node.py:400-404) on a bounded
     sample of the config-2 workload: `sample_rows` rows of bf16 logits, upcast included."""
     import numpy as np
@@ -232,7 +234,7 @@ def cpu_baseline(sample_rows=256, budget_s=12.0):
     oracle.local_compute_logprobs_f32(bits[:8], t[:8], 1.0)   # warm-up
     times = []
     t_end = time.perf_counter() + budget_s
-    while time.perf_counter() < t_end and len(times) < 20:
+    while time.perf_counter() < t_end and len(times) < 40:
         t0 = time.perf_counter()
         oracle.local_compute_logprobs_f32(bits, t, 1.0)
         times.append(time.perf_counter() - t0)
@@ -246,7 +248,7 @@ def cpu_baseline(sample_rows=256, budget_s=12.0):
         threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
         cport.local_compute_logprobs_c(bits[:8], t[:8], 1.0)
         ts = []
-        for _ in range(3):
+        for _ in range(10):
             t0 = time.perf_counter()
             cport.local_compute_logprobs_c(bits, t, 1.0)
             ts.append(time.perf_counter() - t0)
@@ -263,7 +265,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["row", "fused", "decode", "lora"], default=None)
+    ap.add_argument("--only", choices=["row", "fused", "small", "decode", "lora"], default=None)
     ap.add_argument("--row-variant", choices=["both", "mask", "all"], default="both",
                     help="time config 2 with its padding mask, without it, or both (profiling runs pick one)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -295,6 +297,7 @@ def main():
     # the fused step is ~10x longer than a row step: half the launches keep the run short; the clocks
     # still settle (a few tens of milliseconds of back-to-back launches are needed for that)
     fused = bench_fused(dev, max(5, args.steps // 2), max(2, args.warmup // 2)) if args.only in (None, "fused") else None
+    small = bench_fused(dev, args.steps, args.warmup, n=64) if args.only in (None, "small") else None
     decode = bench_decode(dev, args.steps, args.warmup) if args.only in (None, "decode") else None
     lora = bench_lora(dev, max(5, args.steps // 4), max(2, args.warmup // 4)) if args.only in (None, "lora") else None
     cpu = None if args.no_cpu else cpu_baseline()
@@ -343,6 +346,20 @@ def main():
                          "roofline": f["roofline"], "dtype": "f32"})
         else:
             line["fused_lmhead"] = f
+    if small is not None:
+        nbytes = V * small["H"] * 2 + small["tokens"] * small["H"] * 2
+        gbs = nbytes / (small["ms"] * 1e-3) / 1e9
+        d = {"value": small["tokens"] / (small["ms"] * 1e-3), "unit": "token-logprobs/s", "ms_per_step": small["ms"],
+             "dtype": "bf16 x bf16 -> f32",
+             "config": {"workload": "fused lm_head + log-softmax at a decode-step batch: hidden [64,1024] x W [151936,1024] bf16",
+                        "tokens": small["tokens"], "hidden": small["H"], "vocab": V},
+             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                          "traffic": TRAFFIC_FUSED_SMALL_64, "kernel": "fused_lmhead_small_kernel", "bytes_per_launch": nbytes}}
+        if row is None and fused is None:
+            line.update({"value": d["value"], "unit": d["unit"], "ms_per_step": d["ms_per_step"], "config": d["config"],
+                         "roofline": d["roofline"]})
+        else:
+            line["fused_lmhead_decode_batch"] = d
     if decode is not None:
         gbs = decode["bytes"] / (decode["ms"] * 1e-3) / 1e9
         d = {"value": decode["rows"] / (decode["ms"] * 1e-3), "unit": "sampled tokens/s",
