@@ -2,11 +2,13 @@
 """Benchmark of the token-log-prob path on one MI355X.
 
 A step is one pass of the hot path over one batch of synthetic input that is already
-resident in HBM.  The headline workload is BASELINE config 2 (the Qwen3-0.6B GRPO
+resident in HBM.  The headline workload is benchmark configuration 2 (the Qwen3-0.6B GRPO
 ref-logprob shape: bf16 logits [8 x 512, 151936] with a padding mask); the same JSON line
-also carries the unmasked variant and the fused lm_head + log-softmax kernel at config 3.
+also carries the unmasked variant, the fused lm_head + log-softmax kernel at configuration 3
+(4096 tokens) and at a decode-step batch (64 tokens), one decode step's sampler, and the LoRA
+merge of one UpdateWeights request.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only row|fused|decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only row|fused|small|decode|lora]
 
 Prints ONE JSON line on stdout.  Everything else goes to stderr.
 """

@@ -1,4 +1,4 @@
-"""GPU parity at BASELINE's full sizes (configs 2, 4, 5): size-independent properties on every row
+"""GPU parity at the full sizes of the benchmark configurations (2, 4 and 5): size-independent properties on every row
 plus the fp64 oracle on a sample of rows.  Inputs are generated on the GPU with the distributions the
 configs name; sampled rows are copied back bit-exactly for the oracle."""
 import numpy as np

@@ -1,7 +1,7 @@
 """GPU parity of the fused lm_head + log-softmax kernels against the fp64 oracle.
 
 Oracle = exact (fp64) product of the bf16 inputs followed by the closed-form row statistics;
-tolerance 2e-3 abs (bf16 inputs, fp32 accumulation), as BASELINE states for this path.
+tolerance 2e-3 abs (bf16 inputs, fp32 accumulation), the bar stated for this path.
 """
 import numpy as np
 import pytest

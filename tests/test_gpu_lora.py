@@ -158,11 +158,12 @@ def test_merge_rejects_bad_inputs(dev):
     weights.lora_merge([])
 
 
+@pytest.mark.parametrize("n,H", [(333, 512), (48, 1024)])      # the tiled sweep kernel; the small-batch one
 @pytest.mark.parametrize("with_norm,shared_w", [(False, True), (True, True), (False, False), (True, False)])
-def test_grpo_pair_matches_oracle(dev, with_norm, shared_w):
+def test_grpo_pair_matches_oracle(dev, with_norm, shared_w, n, H):
     """Policy and reference hidden states through a shared (or separate) lm_head, optionally pre-norm."""
-    n, H, V = 333, 512, 5000
-    rng = np.random.default_rng(21 + with_norm + 2 * shared_w)
+    V = 5000
+    rng = np.random.default_rng(21 + with_norm + 2 * shared_w + n)
     hp = rand_bits(rng, (n, H), 1.0)
     hr = oracle.bf16_round(oracle.bf16_to_f32(hp) + (rng.standard_normal((n, H)) * 0.05).astype(np.float32))
     wp = rand_bits(rng, (V, H), 0.05)

@@ -1,6 +1,6 @@
 """GPU parity of the row kernel (tome_row_logprob through the Python mirror) against the fp64 oracle.
 
-Tolerances are BASELINE's: 1e-4 abs for fp32 logits, 2e-3 abs for bf16 inputs (the bf16 -> fp32
+Tolerances are the ones stated for this path: 1e-4 abs for fp32 logits, 2e-3 abs for bf16 inputs (the bf16 -> fp32
 upcast is exact, so the bf16 cases are also held to 1e-4); target ids and argmax bit-exact.
 """
 import numpy as np
