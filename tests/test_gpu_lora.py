@@ -51,7 +51,7 @@ def test_merge_bit_exact_on_exact_sums(dev, rows, cols, rank, scale):
 def test_merge_strides_in_place_copy_and_many_jobs(dev):
     rng = np.random.default_rng(11)
     jobs, want, outs = [], [], []
-    for i in range(53):                                    # more jobs than one launch carries
+    for i in range(117):                                   # more jobs than one upload launch carries (56)
         rows, cols, rank = int(rng.integers(1, 90)), 8 * int(rng.integers(1, 140)), int(rng.choice([8, 16, 32, 64, 72]))
         base = rand_bits(rng, (rows, cols), 0.05)
         a, b = exact_bits(rng, (rank, cols)), exact_bits(rng, (rows, rank))
