@@ -83,3 +83,67 @@ def test_sweep_rows_and_sampler(dev, seed):
     assert all(tok[i] in want_idx[i] for i in np.flatnonzero(mb)) and (tok[~mb] == -1).all()
     np.testing.assert_allclose(s.lp.cpu().numpy()[mb], oracle.logprob_rows(x64, np.where(mb, tok, 0), T)[mb], atol=1e-4, rtol=0)
     np.testing.assert_array_equal(s.argmax.cpu().numpy()[mb], oracle.argmax_rows(x64)[mb])
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_sweep_fused_decode_batches(dev, seed):
+    """<= 64 tokens over hidden sizes on and off the streaming kernel's shape rules (K slices of 256 / 512 over 2..8
+    waves), ragged vocabularies (partial last 16-row tile, fewer tiles than CUs), masks, strided hidden states."""
+    rng = np.random.default_rng(5000 + seed)
+    n = int(rng.integers(1, 65))
+    H = int(rng.choice([512, 768, 1024, 1280, 1536, 2048, 2304, 2560, 3072, 4096, 320]))
+    V = int(rng.choice([64, 65, 100, 257, 1000, 4095, 4100, 9001]))
+    T = float(rng.choice([0.5, 0.7, 1.0, 1.6]))
+    kind = str(rng.choice(["none", "random", "prefix"]))
+    pad = int(rng.choice([0, 0, 8, 64]))
+    base = torch.from_numpy(rng.standard_normal((n, H + pad)).astype(np.float32)).to(dev).to(torch.bfloat16)
+    h = base[:, :H]
+    w = torch.from_numpy((rng.standard_normal((V, H)) * rng.uniform(0.01, 0.08)).astype(np.float32)).to(dev).to(torch.bfloat16)
+    t = rng.integers(0, V, size=n).astype(np.int32)
+    m = _mask(rng, n, kind)
+    rv = None if m is None else torch.from_numpy(m).to(dev)
+    r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), T, row_valid=rv, want_lse=True, want_entropy=True,
+                                       want_argmax=True)
+    want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(w), t, T)
+    mb = np.ones(n, bool) if m is None else m.astype(bool)
+    tag = f"n={n} H={H} V={V} {kind} pad={pad}"
+    for name, got in (("lp", r.lp), ("lse", r.lse), ("entropy", r.entropy)):
+        np.testing.assert_allclose(got.cpu().numpy()[mb], want[name][mb], atol=2e-3, rtol=0, err_msg=f"{name} {tag}")
+    clear = mb & ((want["top1"] - want["top2"]) > 1e-2)
+    np.testing.assert_array_equal(r.argmax.cpu().numpy()[clear], want["argmax"][clear], err_msg=tag)
+    assert (r.lp.cpu().numpy()[~mb] == 0).all() and (r.argmax.cpu().numpy()[~mb] == -1).all()
+    lp_only = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), T, row_valid=rv).lp
+    np.testing.assert_allclose(lp_only.cpu().numpy()[mb], want["lp"][mb], atol=2e-3, rtol=0, err_msg=tag)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_sweep_lora_merge(dev, seed):
+    """Random batches of merges (ranks 8..128, ragged rows and columns, strides, base-only jobs) on inputs whose
+    rank-long sums are exact in fp32: bit-exact against the oracle."""
+    from tome_amd import weights
+    rng = np.random.default_rng(6000 + seed)
+    to_dev = lambda b: torch.from_numpy(b.view(np.int16).copy()).to(dev).view(torch.bfloat16)
+    jobs, want, outs = [], [], []
+    for _ in range(int(rng.integers(1, 9))):
+        rows = int(rng.choice([1, 15, 16, 17, 100, 255, 512, 700]))
+        cols = 8 * int(rng.choice([1, 2, 31, 32, 63, 64, 65, 129, 200, 385]))
+        rank = int(rng.choice([8, 16, 24, 32, 40, 64, 96, 128]))
+        scale = float(rng.choice([2.5, 1.0, 0.3, -2.0, 20.0 / 8]))
+        base = oracle.bf16_round((rng.standard_normal((rows, cols)) * 0.05).astype(np.float32))
+        a = oracle.bf16_round((rng.integers(-8, 9, size=(rank, cols)) / 16).astype(np.float32))
+        b = oracle.bf16_round((rng.integers(-8, 9, size=(rows, rank)) / 16).astype(np.float32))
+        spad = 8 * int(rng.integers(0, 3))
+        bt = torch.zeros((rows, cols + spad), device=dev, dtype=torch.bfloat16)
+        bt[:, :cols] = to_dev(base)
+        ot = torch.full((rows, cols + 8), 9.0, device=dev, dtype=torch.bfloat16)
+        if rng.random() < 0.2:
+            jobs.append((bt[:, :cols], ot[:, :cols], None, None, 1.0))
+            want.append(base)
+        else:
+            jobs.append((bt[:, :cols], ot[:, :cols], to_dev(a), to_dev(b), scale))
+            want.append(oracle.lora_merge_bf16(base, a, b, scale))
+        outs.append((ot, cols))
+    weights.lora_merge(jobs)
+    for i, ((ot, cols), w) in enumerate(zip(outs, want)):
+        np.testing.assert_array_equal(bf16_bits_of(ot[:, :cols]), w, err_msg=f"seed {seed} job {i} shape {w.shape}")
+        assert (ot[:, cols:].float() == 9.0).all()
