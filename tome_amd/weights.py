@@ -106,10 +106,35 @@ def lora_merge(jobs: Sequence[MergeJob]) -> None:
     del keep, ws                                   # launches are stream-ordered; torch frees on the same stream
 
 
-def _bf16_from_bytes(raw: bytes, shape: Sequence[int], dev: torch.device) -> torch.Tensor:
-    """``mx.array(np.frombuffer(raw, uint16).reshape(shape)).view(mx.bfloat16)`` (node.py:123-126)."""
-    arr = np.frombuffer(raw, dtype=np.uint16).reshape([int(s) for s in shape])
-    return torch.from_numpy(arr.view(np.int16).copy()).to(dev).view(torch.bfloat16)
+def _upload_lora(entries: Sequence[Tuple[object, float]], dev: torch.device) -> dict:
+    """All adapters of a request in ONE host-to-device copy.
+
+    Each ``LayerUpdate`` is decoded as the reference does - ``np.frombuffer(raw, uint16).reshape(shape)`` viewed
+    as bf16 (node.py:123-126) - with the rank zero-padded to a multiple of 8 (extra terms of the product are exact
+    zeros) and every matrix starting on a 16-byte boundary of one staging array.  Returns
+    ``{id(update): (lora_A [rank, in], lora_B [out, rank])}`` as views of the uploaded buffer.
+    """
+    parts, layout, total = [], {}, 0
+    for up, _ in entries:
+        a = np.frombuffer(up.lora_A, dtype=np.uint16).reshape([int(v) for v in up.shape_A])
+        b = np.frombuffer(up.lora_B, dtype=np.uint16).reshape([int(v) for v in up.shape_B])
+        if a.ndim != 2 or b.ndim != 2 or a.shape[0] != b.shape[1]:
+            raise ValueError(f"lora_A {a.shape} and lora_B {b.shape} do not form a rank decomposition")
+        pad = -a.shape[0] % 8
+        if pad:
+            a = np.concatenate([a, np.zeros((pad, a.shape[1]), np.uint16)], 0)
+            b = np.concatenate([b, np.zeros((b.shape[0], pad), np.uint16)], 1)
+        offs = []
+        for m in (a, b):
+            offs.append((total, m.shape))
+            parts.append((total, m))
+            total += -(-m.size // 8) * 8
+        layout[id(up)] = offs
+    stage = np.zeros(total, dtype=np.uint16)
+    for off, m in parts:
+        stage[off:off + m.size] = m.reshape(-1)
+    buf = torch.from_numpy(stage.view(np.int16)).to(dev).view(torch.bfloat16)
+    return {key: tuple(buf[off:off + sh[0] * sh[1]].view(sh) for off, sh in offs) for key, offs in layout.items()}
 
 
 def apply_weight_update(policy_layers: Sequence, reference_layers: Sequence, updates: Sequence, *,
@@ -131,10 +156,16 @@ def apply_weight_update(policy_layers: Sequence, reference_layers: Sequence, upd
 
     jobs: List[MergeJob] = []
     rebuilt = 0
+    uploaded: dict = {}                                              # device -> adapters of that device's layers
 
     def lora(entry, dev):
+        if dev not in uploaded:
+            mine = [e for li, d in layer_deltas.items() for e in d.values()
+                    if reference_layers[li].self_attn.qkv_proj.weight.device == dev]
+            uploaded[dev] = _upload_lora(mine, dev)
         up, scale = entry
-        return _bf16_from_bytes(up.lora_A, up.shape_A, dev), _bf16_from_bytes(up.lora_B, up.shape_B, dev), scale
+        a, b = uploaded[dev][id(up)]
+        return a, b, scale
 
     for layer_idx, deltas in layer_deltas.items():                   # node.py:132-151
         ref_layer, target = reference_layers[layer_idx], policy_layers[layer_idx]
