@@ -66,7 +66,9 @@ Pinning (tests/test_oracle.py):
                             is pinned by closed forms (zero A -> the base bit for bit,
                             rank-1 outer product, B selecting rows of A, linearity in
                             scale on exactly representable inputs), brute-force loops
-                            with math.fsum, and numpy's float64 matmul; the
+                            with math.fsum, numpy's float64 matmul and committed golden
+                            vectors from exact rational arithmetic
+                            (tests/golden/make_lora_golden.py); the
                             bookkeeping (last update wins, scale 0 -> 1.0, qkv_proj
                             over q/k/v, missing q/k/v slices revert to the base,
                             non-cumulative, untouched layers kept) by known-answer

@@ -197,3 +197,15 @@ def test_grpo_pair_matches_oracle(dev, with_norm, shared_w, n, H):
                                            w_ref=to_dev(wr, dev))
         for x, y in zip(dual, pair):
             np.testing.assert_array_equal(x.cpu().numpy(), y.cpu().numpy())
+
+
+@pytest.mark.parametrize("name", ["m0", "m1", "m2", "m3"])
+def test_merge_matches_golden_vectors(dev, name):
+    """The committed vectors (exact rational arithmetic, tests/golden/make_lora_golden.py); ranks 12 and 4 are
+    zero-padded by the wrapper."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "lora_golden.npz"))
+    base, a, b = g[f"{name}_base"], g[f"{name}_a"], g[f"{name}_b"]
+    out = torch.empty(base.shape, device=dev, dtype=torch.bfloat16)
+    weights.lora_merge([(to_dev(base, dev), out, to_dev(a, dev), to_dev(b, dev), float(g[f"{name}_scale"]))])
+    np.testing.assert_array_equal(bf16_bits_of(out), g[f"{name}_out"])

@@ -216,3 +216,12 @@ def test_servicer_reports_failure_instead_of_raising(patched, monkeypatch):
     assert not r.success
     ok = svc.update_weights(types.SimpleNamespace(updates=[]))             # an empty request still bumps the version
     assert ok.success and ok.policy_version == 2
+
+
+@pytest.mark.parametrize("name", ["m0", "m1", "m2", "m3"])
+def test_oracle_merge_matches_golden_vectors(name):
+    """tests/golden/lora_golden.npz: exact rational arithmetic + an independent bf16 rounding (make_lora_golden.py)."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "lora_golden.npz"))
+    got = oracle.lora_merge_bf16(g[f"{name}_base"], g[f"{name}_a"], g[f"{name}_b"], float(g[f"{name}_scale"]))
+    np.testing.assert_array_equal(got, g[f"{name}_out"])
