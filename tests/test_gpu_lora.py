@@ -209,3 +209,47 @@ def test_merge_matches_golden_vectors(dev, name):
     out = torch.empty(base.shape, device=dev, dtype=torch.bfloat16)
     weights.lora_merge([(to_dev(base, dev), out, to_dev(a, dev), to_dev(b, dev), float(g[f"{name}_scale"]))])
     np.testing.assert_array_equal(bf16_bits_of(out), g[f"{name}_out"])
+
+
+def test_update_weights_at_qwen3_0_6b_scale(dev):
+    """All 84 matrices of a Qwen3-0.6B request in one call (the benchmark's workload), checked by properties that do
+    not need the CPU oracle at this size: a torch fp32 restatement with the same three roundings (bit-equal except
+    where fp32 summation order flips the product's rounding), base-only jobs returning the base, and a second
+    identical call changing nothing (non-cumulative)."""
+    g = torch.Generator(device=dev).manual_seed(7)
+    shapes = [(4096, 1024), (6144, 1024), (1024, 3072)]
+    jobs, bases, outs, loras = [], [], [], []
+    for i in range(28 * 3):
+        rows, cols = shapes[i % 3]
+        base = (torch.randn((rows, cols), device=dev, generator=g) * 0.02).to(torch.bfloat16)
+        out = torch.empty_like(base)
+        a = (torch.randn((8, cols), device=dev, generator=g) * 0.05).to(torch.bfloat16)
+        b = (torch.randn((rows, 8), device=dev, generator=g) * 0.05).to(torch.bfloat16)
+        if i % 11 == 5:
+            jobs.append((base, out, None, None, 1.0))
+            loras.append(None)
+        else:
+            jobs.append((base, out, a, b, 2.5))
+            loras.append((a, b))
+        bases.append(base)
+        outs.append(out)
+    weights.lora_merge(jobs)
+    first = [o.clone() for o in outs]
+    weights.lora_merge(jobs)
+    differ = total = 0
+    for base, out, again, lo in zip(bases, outs, first, loras):
+        assert torch.equal(out, again)
+        if lo is None:
+            assert torch.equal(out.view(torch.int16), (base.float() + 0.0).to(torch.bfloat16).view(torch.int16))
+            continue
+        a, b = lo
+        d = (b.float() @ a.float()).to(torch.bfloat16).float()
+        want = (base.float() + (2.5 * d).to(torch.bfloat16).float()).to(torch.bfloat16)
+        ne = out.view(torch.int16) != want.view(torch.int16)
+        differ += int(ne.sum())
+        total += ne.numel()
+        if ne.any():             # one flipped step of the product moves the scaled delta by up to 2^-6 of itself,
+            gap = (out.float() - want.float()).abs()[ne]          # the sum then rounds once more
+            bound = (2.0 ** -6 * (2.5 * d).abs() + 2.0 ** -7 * want.float().abs())[ne]
+            assert (gap <= bound).all()
+    assert differ <= total * 1e-4, f"{differ} of {total} elements differ from the torch restatement"
