@@ -267,10 +267,11 @@ def test_norm_lmhead_matches_oracle(dev, n, H, V, masked):
 @pytest.mark.parametrize("n,H,V,masked", [
     (1, 1024, 151936, False), (16, 1024, 40000, True), (17, 1024, 8191, False), (64, 1024, 151936, True),
     (33, 2048, 30001, False), (64, 2048, 12345, True), (9, 4096, 20000, False), (32, 4096, 33000, True),
-    (20, 2560, 9000, False), (5, 512, 7000, False), (64, 1536, 5000, False), (48, 1024, 70, False)])
+    (20, 2560, 9000, False), (5, 512, 7000, False), (64, 1536, 5000, False), (48, 1024, 70, False),
+    (65, 1024, 5001, False), (100, 1024, 30000, True), (128, 1024, 151936, False), (128, 1024, 200, True)])
 def test_fused_small_batch_kernel(dev, n, H, V, masked):
-    """Decode-sized batches (<= 64 tokens) take the streaming kernel with K split across waves (where the shape
-    rules allow it; the other shapes here fall back to the tiled kernel) - same bar either way."""
+    """Decode-sized batches (<= 64 tokens; <= 128 at H = 1024) take the streaming kernel with K split across waves
+    (where the shape rules allow it; the other shapes here fall back to the tiled kernel) - same bar either way."""
     rng = np.random.default_rng(n * 31 + H + V)
     h, w, t = _inputs(dev, n, H, V, n * 31 + H + V, w_scale=0.05)
     valid = (rng.random(n) < 0.7).astype(np.int32) if masked else np.ones(n, dtype=np.int32)

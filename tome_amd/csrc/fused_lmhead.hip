@@ -744,13 +744,15 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 //   * Per tile the waves' partial sums (16 rows x 16*NBT tokens, MFMA layout) meet in LDS; wave j sums
 //     them in wave order and folds token block j into its online-softmax state.  One barrier per tile:
 //     the buffer of tile t is rewritten at tile t + 2, after the barrier of tile t + 1, which the
-//     folding waves only reach once tile t is folded.
+//     folding waves only reach once tile t is folded.  (Eight token blocks - 65..128 tokens, K slices of
+//     128 on 8 waves, H = 1024 only - use one buffer and a second barrier: two would not fit the LDS.)
 //   * One partial per (token, workgroup); the combine kernel is shared with the other paths.
 // ===============================================================================================
 template <bool ENT, bool AMAX, int NBT, int KSTEPS>
 __global__ __launch_bounds__(512) void fused_lmhead_small_kernel(FusedArgs a) {
   extern __shared__ __attribute__((aligned(16))) char small_mem[];  // [2][waves][NBT][64 lanes] f32x4, then [waves] 4 KB tiles
-  constexpr int kBuf = 16 / KSTEPS;                                 // tile buffers in flight: 2 or 1
+  constexpr int kBuf = NBT == 8 ? 2 : 16 / KSTEPS;                  // tile buffers in flight (registers): 16 loads, 8 with 8 token blocks
+  constexpr int kRed = NBT == 8 ? 1 : 2;                            // reduction buffers (LDS)
   const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
   if (n_valid <= 0) return;
   const int lane = threadIdx.x & 63;
@@ -797,7 +799,7 @@ __global__ __launch_bounds__(512) void fused_lmhead_small_kernel(FusedArgs a) {
     row = row < a.V ? row : a.V - 1;
     return a.weight + (int64_t)row * a.weight_stride_b + wave * (KSTEPS * 64) + lc * 16;
   };
-  char* stage = small_mem + (size_t)2 * n_waves * NBT * 1024 + wave * 4096;
+  char* stage = small_mem + (size_t)kRed * n_waves * NBT * 1024 + wave * 4096;
   u32x4 wb[kBuf][kUnits][4];
 #pragma unroll
   for (int b = 0; b < kBuf && t0 < t1; ++b) {
@@ -846,16 +848,17 @@ __global__ __launch_bounds__(512) void fused_lmhead_small_kernel(FusedArgs a) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the next unit overwrites what was just read
         __builtin_amdgcn_wave_barrier();
       }
-      char* red = small_mem + (size_t)(((t & 1) * n_waves + wave) * NBT) * 1024 + lane * 16;
+      char* red = small_mem + (size_t)(((t & (kRed - 1)) * n_waves + wave) * NBT) * 1024 + lane * 16;
 #pragma unroll
       for (int j = 0; j < NBT; ++j) *reinterpret_cast<f32x4v*>(red + j * 1024) = acc[j];
       __syncthreads();
       if (wave < NBT) {
         f32x4v sum[1][1] = {{f32x4v{0.f, 0.f, 0.f, 0.f}}};
-        const char* src = small_mem + (size_t)((t & 1) * n_waves * NBT + wave) * 1024 + lane * 16;
+        const char* src = small_mem + (size_t)((t & (kRed - 1)) * n_waves * NBT + wave) * 1024 + lane * 16;
         for (int w = 0; w < n_waves; ++w) sum[0][0] += *reinterpret_cast<const f32x4v*>(src + (size_t)w * NBT * 1024);
         fold_tile16<ENT, AMAX, 1, 1>(sum, st, tx, tgt, t * 16, g, t * 16 + 16 > a.V, a.V, a.scale);
       }
+      if constexpr (kRed == 1) __syncthreads();  // one buffer: the next tile's sums wait for this fold
     }
   }
   // One partial per (token, workgroup): part index = workgroup id.
@@ -1121,20 +1124,26 @@ static int small_wg_count() {
 }
 
 // Shape rules of the small-batch kernel: <= 64 tokens, K split over 2..8 waves in slices of 256 or 512
-// (slices of 128 on twice the waves measured 2 us slower at H = 1024).
+// (slices of 128 on twice the waves measured 2 us slower at H = 1024); 65..128 tokens at H = 1024 only.
 static bool small_shape(int64_t n_tokens, int64_t H, int64_t V, int& nbt, int& ksteps, int& waves) {
-  if (n_tokens > 64 || V < 64) return false;
+  if (n_tokens > 128 || V < 64) return false;
+  if (n_tokens > 64) {  // eight token blocks: the B fragments only fit with K slices of 128, on exactly 8 waves
+    nbt = 8;
+    ksteps = 4;
+    waves = 8;
+    return H == 1024;
+  }
   nbt = n_tokens <= 16 ? 1 : (n_tokens <= 32 ? 2 : 4);
   if (H % 256 == 0 && H / 256 <= 8 && H / 256 >= 2) {
     ksteps = 8;
     waves = (int)(H / 256);
-  } else if (H % 512 == 0 && H / 512 <= 8 && nbt <= 2) {
+  } else if (H % 512 == 0 && H / 512 <= 8 && H / 512 >= 2 && nbt <= 2) {
     ksteps = 16;
     waves = (int)(H / 512);
   } else {
     return false;
   }
-  if (ksteps == 8 && nbt == 2) nbt = 4;  // instantiated token-block counts: 1 and 4 (K 256), 1 and 2 (K 512)
+  if (ksteps == 8 && nbt == 2) nbt = 4;  // instantiated token-block counts: 1 and 4 (K 256), 1 and 2 (K 512), 8 (K 128)
   return waves >= nbt;
 }
 
@@ -1151,12 +1160,12 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   p.n_vtiles = 0;
   if (p.kind == kSmall) {
     // One partial per (token, workgroup); one workgroup per CU, at most 512.
-    p.bt = 64;
+    p.bt = 128;
     p.bv = 16;
     p.slots = 1;     // only feed the schedule that the compaction kernel writes and this path ignores
     p.n_vtiles = 1;
     p.grid = 0;
-    p.max_records = (size_t)64 * 512;
+    p.max_records = (size_t)128 * 512;
     return p;
   }
   p.bt = p.kind == kGeneric ? kBT : k2BT;   // the DMA path has a 256 x 256 tile
@@ -1207,7 +1216,7 @@ static int launch_small(const FusedArgs& a, int waves, hipStream_t stream) {
   const int n_tiles = (a.V + 15) / 16;
   if (n_wg > n_tiles) n_wg = n_tiles & ~1;  // no empty vocab ranges
   if (n_wg < 2) return 0;
-  const size_t lds = (size_t)2 * waves * NBT * 1024 + (size_t)waves * 4096;
+  const size_t lds = (size_t)(NBT == 8 ? 1 : 2) * waves * NBT * 1024 + (size_t)waves * 4096;
   static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
   if (!attr_set && lds > 65536) {
     allow_big_lds(&fused_lmhead_small_kernel<ENT, AMAX, NBT, KSTEPS>, 2 * 8 * 4 * 1024 + 8 * 4096);
@@ -1227,7 +1236,8 @@ static int launch_main(const FusedArgs& a, const FusedPlan& plan, bool want_argm
     const int w = plan.small_waves;
 #define TOME_SMALL(NBT, KS)                                                 \
   n = want_argmax ? launch_small<ENT, true, NBT, KS>(a, w, stream) : launch_small<ENT, false, NBT, KS>(a, w, stream)
-    if (plan.small_ksteps == 8 && plan.small_nbt == 1) TOME_SMALL(1, 8);
+    if (plan.small_nbt == 8) TOME_SMALL(8, 4);
+    else if (plan.small_ksteps == 8 && plan.small_nbt == 1) TOME_SMALL(1, 8);
     else if (plan.small_ksteps == 8) TOME_SMALL(4, 8);
     else if (plan.small_nbt == 1) TOME_SMALL(1, 16);
     else TOME_SMALL(2, 16);
