@@ -33,7 +33,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 TRAFFIC_ROW_MASKED = 716.4e6 + 0.13e6
 TRAFFIC_ROW_ALL = 1245.0e6 + 0.13e6
 TRAFFIC_FUSED_CFG3 = 1847e6 + 6.8e6
-TRAFFIC_DECODE_64 = 39.4e6 + 0.42e6 + 0.40e6   # sampler: main-kernel fetch, combine fetch, partials written
+TRAFFIC_DECODE_64 = 39.2e6 + 0.30e6 + 0.23e6   # sampler: main-kernel fetch, combine fetch, partials written
 TRAFFIC_FUSED_SMALL_64 = 326.0e6 + 0.52e6      # sweep kernel: fetch + partials written (profiles/fused_lmhead_small_kernel_decode_64tokens.txt)
 TRAFFIC_LORA_06B = 812.1e6 + 763.4e6            # merge kernel: fetch + write (profiles/lora_merge_kernel_qwen3_0.6b_update.txt)
 

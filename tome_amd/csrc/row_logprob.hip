@@ -203,12 +203,14 @@ static hipError_t dispatch_flags(const RowArgs& a, int64_t rows, hipStream_t str
   return launch_row<T, VECTOR, false, false>(a, rows, stream);
 }
 
-// How many workgroups share a row.  Large batches use one workgroup per row; small ones
-// (decode steps, the 64-row CPU-comparison case) are split so that at least ~8 workgroups
-// per CU are in flight, as long as every split keeps a few loads per lane.
+// How many workgroups share a row.  From 512 rows on one workgroup per row; smaller batches (decode steps,
+// the 64-row CPU-comparison case) are split so that ~2 workgroups per CU are in flight, as long as every
+// split keeps a few loads per lane.  Measured: aiming at 512 to 2048 workgroups is equal within 0.5 us for
+// 32-256 rows, and 512 spares the 512- and 1024-row batches the combine launch (27.0 against 30.6 us,
+// 50.3 against 52.7 us); 3072 and more are slower everywhere.
 int row_splits_for(int64_t rows, int64_t V, int vec) {
   const int64_t units = V / vec;
-  const int64_t want_wgs = 2048;
+  const int64_t want_wgs = 512;
   int64_t s = (want_wgs + rows - 1) / rows;
   const int64_t max_by_work = units / (2 * kRowWG);  // >= 2 loads per lane per split
   if (s > max_by_work) s = max_by_work;
