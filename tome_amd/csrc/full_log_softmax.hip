@@ -24,10 +24,11 @@ struct FullArgs {
 
 __device__ __forceinline__ float bf16_rt(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
+// Two elements: round the scaled logits to bf16, subtract, round again (v_cvt_pk_bf16_f32 twice; the
+// software rounding this replaces cost more VALU time than the memory stream left room for).
 __device__ __forceinline__ uint32_t sub_pack_bf16(uint32_t u, float inv_temp, float lse_t) {
-  const float lo = bf16_rt(__fsub_rn(bf16_rt(__fmul_rn(bf16_lo(u), inv_temp)), lse_t));
-  const float hi = bf16_rt(__fsub_rn(bf16_rt(__fmul_rn(bf16_hi(u), inv_temp)), lse_t));
-  return (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
+  const uint32_t z = pack_bf16(__fmul_rn(bf16_lo(u), inv_temp), __fmul_rn(bf16_hi(u), inv_temp));
+  return pack_bf16(__fsub_rn(bf16_lo(z), lse_t), __fsub_rn(bf16_hi(z), lse_t));
 }
 
 template <bool BF16, bool VECTOR>
@@ -106,8 +107,11 @@ hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t
   a.out_stride = out_stride;
   a.inv_temp = 1.0f / temperature;  // the reference multiplies by 1/temp (model.py:27)
   const int64_t units = V / (vector_ok ? vec : 1);
-  int64_t chunks = (4096 + rows - 1) / rows;
-  const int64_t by_work = units / kFullWG;
+  // Many short workgroups stream a read + write mix best (measured: aiming at 65536 workgroups instead of 4096
+  // takes 512 x 151936 fp32 from 165 to 150 us and 4096 x 151936 bf16 from 655 to 633 us, both passes included),
+  // as long as each still issues its four loads per lane.
+  int64_t chunks = (65536 + rows - 1) / rows;
+  const int64_t by_work = units / (kFullUnroll * kFullWG);
   if (chunks > by_work) chunks = by_work;
   if (chunks < 1) chunks = 1;
   a.chunks = (int)chunks;
