@@ -54,6 +54,16 @@ def test_signatures_mirror_the_reference():
     assert list(p) == ["self", "prompts", "results", "G", "temperature"] and p["temperature"].default == 1.0
     # node.py:58  max_ref_batch_size=32
     assert inspect.signature(tome_amd.RefLogprobServicer.__init__).parameters["max_ref_batch_size"].default == 32
+    # node.py:102-106  async UpdateWeights(self, request, context) -> WeightUpdateResponse(success, policy_version)
+    m = tome_amd.WeightUpdateServicer.UpdateWeights
+    assert inspect.iscoroutinefunction(m) and list(inspect.signature(m).parameters)[:3] == ["self", "request", "context"]
+    # inference.proto:68-81  LayerUpdate / WeightUpdateResponse field names
+    import dataclasses
+    assert [f.name for f in dataclasses.fields(tome_amd.LayerUpdate)] == [
+        "layer_idx", "param_name", "lora_A", "lora_B", "shape_A", "shape_B", "lora_scale"]
+    assert [f.name for f in dataclasses.fields(tome_amd.WeightUpdateResponse)] == ["success", "policy_version"]
+    # node.py:894  _sample_token's top_k = 20
+    assert inspect.signature(tome_amd.sample_tokens).parameters["top_k"].default == 20
 
 
 def test_temperature_validation():
