@@ -18,10 +18,10 @@
 //     (max, sum 2^(y-m), sum y 2^(y-m)) states.  Two kernels share this shape; a third,
 //     fused_lmhead_small_kernel (<= 64 tokens, W streamed once, K split across waves), is
 //     described where it is defined:
-//       fused_lmhead_dma_kernel  (H % 64 == 0, more than 128 tokens) 512 lanes, 256 x 256 tile,
+//       fused_lmhead_dma_kernel  (H % 64 == 0) 512 lanes, 256 vocab rows x 256 / 128 / 64 tokens,
 //                                16x16x32 MFMA, K slabs DMA'd into LDS - described at the kernel;
-//       fused_lmhead_kernel      (any H % 8, short batches) 256 lanes, 256 x 128 tile, 32x32x16
-//                                MFMA, 64-wide slabs staged through registers into padded LDS.
+//       fused_lmhead_kernel      (any H % 8) 256 lanes, 256 x 128 tile, 32x32x16 MFMA, 64-wide
+//                                slabs staged through registers into padded LDS.
 //   * The vocab axis is split over workgroups (fused_schedule); each writes one partial per
 //     (token, split, vocab-wave) and fused_combine_kernel merges them deterministically.
 //   * Masked tokens are compacted first (compact_rows_kernel); token tiles are built from
@@ -514,16 +514,21 @@ __device__ __forceinline__ void write_partials16(RowStat (&st)[NBT], float (&tx)
 //     8*(r&1) .. +7, so chunk c of row r is stored at chunk position c ^ ((r >> 1) & 7); the
 //     lane that DMA-writes position p of row r fetches global chunk p ^ ((r >> 1) & 7).
 // ===============================================================================================
-constexpr int k2BV = 256, k2BT = 256, k2WG = 512;
+//
+// The token tile is a template parameter: NBT = 4 token blocks per wave (256 tokens per workgroup) is the
+// shape described above and the one the MFMA/DMA interleave is tuned for; NBT = 2 and 1 (128 and 64
+// tokens) serve batches of up to one such tile, where W is streamed once and the kernel is bound by
+// that stream: they do the MFMA work of 128 or 64 tokens instead of 256 per slab of W.
+constexpr int k2BV = 256, k2WG = 512;
 constexpr int k2BK = 64;
 constexpr int k2RowBytes = k2BK * 2;                     // 128: one cache line
-constexpr int k2SlabBytes = (k2BV + k2BT) * k2RowBytes;  // 65536
 constexpr int k2Slabs = 2;
-constexpr int k2LdsTotal = k2Slabs * k2SlabBytes;        // 131072
-constexpr int k2Loads = k2BV * (k2RowBytes / 16) / k2WG; // DMA instructions per lane, operand and slab (4)
-constexpr int k2DmaPerSlab = 2 * k2Loads;                // DMA instructions per slab and wave (8)
-constexpr int k2NBV = kWaveV / 16, k2NBT = kWaveT / 16;  // 16x16 blocks per wave tile: 8 x 4
-static_assert(k2DmaPerSlab == 8 && k2NBV == 8 && k2NBT == 4, "the MFMA/DMA interleave is written for this shape");
+constexpr int k2Loads = k2BV * (k2RowBytes / 16) / k2WG; // DMA instructions per lane and slab for W (4)
+constexpr int k2NBV = kWaveV / 16;                       // 16x16 vocab blocks per wave tile: 8
+static_assert(k2Loads == 4 && k2NBV == 8, "the MFMA/DMA interleave is written for this shape");
+constexpr int dma_tile_tokens(int nbt) { return nbt * 64; }                                   // 4 token waves x nbt x 16
+constexpr int dma_slab_bytes(int nbt) { return (k2BV + dma_tile_tokens(nbt)) * k2RowBytes; }  // 65536 at nbt = 4
+constexpr int dma_lds_bytes(int nbt) { return k2Slabs * dma_slab_bytes(nbt); }                // 131072 at nbt = 4
 
 __device__ __forceinline__ void dma16(const char* gptr, char* lds_wave_base) {
   __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(gptr),
@@ -540,9 +545,15 @@ __device__ __forceinline__ void pair_reads() {
   }
 }
 
-template <bool ENT, bool AMAX>
+template <bool ENT, bool AMAX, int NBT>
 __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int k2NBT = NBT;                        // 16-token blocks per wave
+  constexpr int k2BT = dma_tile_tokens(NBT);        // tokens per workgroup
+  constexpr int kWaveTok = NBT * 16;                // tokens per wave
+  constexpr int k2SlabBytes = dma_slab_bytes(NBT);
+  constexpr int kBLoads = NBT;                      // DMA instructions per lane and slab for the hidden rows
+  constexpr int k2DmaPerSlab = k2Loads + kBLoads;   // 8 at NBT = 4
 
   const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
   const FusedSchedule sch = a.sched_dev ? *a.sched_dev : a.sched;
@@ -563,7 +574,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   const int dr = lane >> 3;                                   // row inside the 8-row group
   const int dc = (lane & 7) ^ (4 * (wave & 1) + (dr >> 1));   // global chunk: position ^ ((row >> 1) & 7)
   const char* pa[k2Loads];  // next W slab to request, per DMA instruction
-  const char* pb[k2Loads];  // next hidden slab
+  const char* pb[kBLoads];  // next hidden slab
   auto point_a = [&](int vt) {  // rows past V (last tile only) read the last row; masked in the epilogue
 #pragma unroll
     for (int j = 0; j < k2Loads; ++j) {
@@ -574,7 +585,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   };
   point_a(vt0);
 #pragma unroll
-  for (int j = 0; j < k2Loads; ++j) {
+  for (int j = 0; j < kBLoads; ++j) {
     int p = t0 + (j * 8 + wave) * 8 + dr;
     p = p < n_valid ? p : n_valid - 1;
     const int tok = a.hidden_index ? a.hidden_index[p] : p;
@@ -589,7 +600,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   for (int bt = 0; bt < k2NBT; ++bt) {
     st[bt] = stat_identity();
     tx[bt] = -INFINITY;
-    const int p = t0 + wave_t * kWaveT + bt * 16 + l16;
+    const int p = t0 + wave_t * kWaveTok + bt * 16 + l16;
     int t = -1;
     if (p < n_valid) t = a.targets[a.row_index ? a.row_index[p] : p];
     tgt[bt] = (t >= 0 && t < a.V) ? t : -1;
@@ -598,7 +609,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   // ---- fragment read offsets inside a slab (swizzled): lane group g reads chunk 4*ks + g ----------
   const int swz = (g ^ ((l16 >> 1) & 7)) * 16;  // sub-step k0; k1 is this ^ 64
   const int rdA = (wave_v * kWaveV + l16) * k2RowBytes + swz;
-  const int rdB = k2BV * k2RowBytes + (wave_t * kWaveT + l16) * k2RowBytes + swz;
+  const int rdB = k2BV * k2RowBytes + (wave_t * kWaveTok + l16) * k2RowBytes + swz;
 
   const int nk = a.H / k2BK;
   const int n_steps = (vt1 - vt0) * nk;
@@ -619,15 +630,14 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     if (issued >= n_steps) return;  // the stream stays on the last slab
     if (++i_kt < nk) {
 #pragma unroll
-      for (int j = 0; j < k2Loads; ++j) {
-        pa[j] += k2RowBytes;
-        pb[j] += k2RowBytes;
-      }
+      for (int j = 0; j < k2Loads; ++j) pa[j] += k2RowBytes;
+#pragma unroll
+      for (int j = 0; j < kBLoads; ++j) pb[j] += k2RowBytes;
     } else {
       i_kt = 0;
       ++i_vt;
 #pragma unroll
-      for (int j = 0; j < k2Loads; ++j) pb[j] -= slab_rewind;
+      for (int j = 0; j < kBLoads; ++j) pb[j] -= slab_rewind;
       if (i_vt < vt1) point_a(i_vt);
     }
   };
@@ -650,7 +660,10 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
     issue_done();
   }
-  asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // slab 0 has landed (this wave's share)
+  // slab 0 has landed (this wave's share): only the requests of slab 1 may still be in flight
+  if constexpr (k2DmaPerSlab == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else if constexpr (k2DmaPerSlab == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
   __syncthreads();
 
   bf16x8 fa_lo[4], fa_hi[4], fb0[k2NBT], fb1[k2NBT];
@@ -683,16 +696,16 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     __builtin_amdgcn_sched_barrier(0);
     read_a(step, 0, 4, fa_hi);
     mfma_half(0, fa_lo, fb0, fresh);
-    pair_reads<2, 4>();
+    if constexpr (NBT == 4) pair_reads<2, 4>();
     __builtin_amdgcn_sched_barrier(0);
     read_a(step, 1, 0, fa_lo);
     read_b(step, 1, fb1);
     mfma_half(4, fa_hi, fb0, fresh);
-    pair_reads<2, 8>();
+    if constexpr (NBT == 4) pair_reads<2, 8>();
     __builtin_amdgcn_sched_barrier(0);
     read_a(step, 1, 4, fa_hi);
     mfma_half(0, fa_lo, fb1, std::false_type{});
-    pair_reads<2, 4>();
+    if constexpr (NBT == 4) pair_reads<2, 4>();
     __builtin_amdgcn_sched_barrier(0);
     // This wave has read all it needs of slab `step` and its share of slab step+1 has landed; after
     // the (fence-less) barrier both hold for everyone.
@@ -707,11 +720,13 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 #pragma unroll
     for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
     mfma_half(4, fa_hi, fb1, std::false_type{});
-    pair_reads<1, 8>();
+    if constexpr (NBT == 4) {
+      pair_reads<1, 8>();
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM (DMA request)
+      for (int q = 0; q < 8; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM (DMA request)
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
     issue_done();
@@ -726,7 +741,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no request may outlive the workgroup's LDS
 
-  write_partials16(st, tx, a.partials, t0 + wave_t * kWaveT, n_valid, split * kPartsPerSplit + wave_v,
+  write_partials16(st, tx, a.partials, t0 + wave_t * kWaveTok, n_valid, split * kPartsPerSplit + wave_v,
                    sch.n_splits * kPartsPerSplit, l16, g, a.scale);
 }
 
@@ -1088,13 +1103,14 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
 }
 
 // ---- host side -----------------------------------------------------------------------------------
-// The DMA kernel needs whole 64-wide K slabs and pays for 256-token tiles; short batches and ragged H
-// go to the generic kernel.
+// The DMA kernel needs whole 64-wide K slabs (ragged H goes to the generic kernel); its token tile shrinks
+// with the batch.  Decode-sized batches whose hidden states fit the waves' registers take the streaming kernel.
 
 enum FusedKind { kGeneric = 0, kDma = 1, kSmall = 2 };
 
 struct FusedPlan {
   FusedKind kind;
+  int dma_nbt;                               // kDma only: token blocks per wave (4, 2 or 1: 256, 128 or 64 tokens per tile)
   int small_nbt, small_ksteps, small_waves;  // kSmall only
   int bt, bv, slots, n_vtiles;
   int grid;            // workgroups to launch: the most any number of valid tokens can ask for
@@ -1151,7 +1167,8 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   FusedPlan p;
   p.kind = kGeneric;
   p.small_nbt = p.small_ksteps = p.small_waves = 0;
-  if (n_tokens > kBT && H % k2BK == 0) p.kind = kDma;
+  p.dma_nbt = n_tokens > 128 ? 4 : (n_tokens > 64 ? 2 : 1);
+  if (H % k2BK == 0) p.kind = kDma;
   if (small_shape(n_tokens, H, V, p.small_nbt, p.small_ksteps, p.small_waves)) p.kind = kSmall;
   if (const char* ov = getenv("TOME_FUSED_KERNEL")) {  // tuning knob: force a path where its shape rules allow
     if (ov[0] == 'g') p.kind = kGeneric;
@@ -1168,9 +1185,11 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
     p.max_records = (size_t)128 * 512;
     return p;
   }
-  p.bt = p.kind == kGeneric ? kBT : k2BT;   // the DMA path has a 256 x 256 tile
+  p.bt = p.kind == kGeneric ? kBT : dma_tile_tokens(p.dma_nbt);   // the DMA path: 256 vocab rows x 256, 128 or 64 tokens
   p.bv = p.kind == kGeneric ? kBV : k2BV;
-  p.slots = p.kind == kGeneric ? 512 : 256;  // resident workgroups on 256 CUs: 2 per CU, or 1 (128 KB LDS)
+  // resident workgroups on 256 CUs: 2 per CU, or 1 for the DMA path (80-128 KB of LDS; two 64-token workgroups of 80 KB
+  // per CU measured slower than one: 288 against 277 us at 64 x 4096)
+  p.slots = p.kind == kGeneric ? 512 : 256;
   p.n_vtiles = (int)((V + p.bv - 1) / p.bv);
   p.grid = 0;
   p.max_records = 0;
@@ -1200,14 +1219,21 @@ size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weigh
   return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, H, V) + normed_bytes(n_tokens, H, with_norm);
 }
 
-template <bool ENT, bool AMAX>
-static void launch_dma(const FusedArgs& a, int grid, hipStream_t stream) {
+template <bool ENT, bool AMAX, int NBT>
+static void launch_dma_nbt(const FusedArgs& a, int grid, hipStream_t stream) {
   static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
   if (!attr_set) {
-    allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX>, k2LdsTotal);
+    allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX, NBT>, dma_lds_bytes(NBT));
     attr_set = true;
   }
-  hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX>), dim3((unsigned)grid), dim3(k2WG), k2LdsTotal, stream, a);
+  hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX, NBT>), dim3((unsigned)grid), dim3(k2WG), dma_lds_bytes(NBT), stream,
+                     a);
+}
+template <bool ENT, bool AMAX>
+static void launch_dma(const FusedArgs& a, int nbt, int grid, hipStream_t stream) {
+  if (nbt == 4) launch_dma_nbt<ENT, AMAX, 4>(a, grid, stream);
+  else if (nbt == 2) launch_dma_nbt<ENT, AMAX, 2>(a, grid, stream);
+  else launch_dma_nbt<ENT, AMAX, 1>(a, grid, stream);
 }
 
 template <bool ENT, bool AMAX, int NBT, int KSTEPS>
@@ -1245,8 +1271,8 @@ static int launch_main(const FusedArgs& a, const FusedPlan& plan, bool want_argm
     return n >= 2 ? n : -1;
   }
   if (plan.kind == kDma) {
-    if (want_argmax) launch_dma<ENT, true>(a, plan.grid, stream);
-    else launch_dma<ENT, false>(a, plan.grid, stream);
+    if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.grid, stream);
+    else launch_dma<ENT, false>(a, plan.dma_nbt, plan.grid, stream);
   } else {
     hipLaunchKernelGGL(fused_lmhead_kernel<ENT>, dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
   }
