@@ -522,13 +522,13 @@ __device__ __forceinline__ void write_partials16(RowStat (&st)[NBT], float (&tx)
 constexpr int k2BV = 256, k2WG = 512;
 constexpr int k2BK = 64;
 constexpr int k2RowBytes = k2BK * 2;                     // 128: one cache line
-constexpr int k2Slabs = 2;
+constexpr int dma_slabs(int nbt) { return nbt == 4 ? 2 : 3; }  // slab buffers: as many as fit the 160 KB of LDS
 constexpr int k2Loads = k2BV * (k2RowBytes / 16) / k2WG; // DMA instructions per lane and slab for W (4)
 constexpr int k2NBV = kWaveV / 16;                       // 16x16 vocab blocks per wave tile: 8
 static_assert(k2Loads == 4 && k2NBV == 8, "the MFMA/DMA interleave is written for this shape");
 constexpr int dma_tile_tokens(int nbt) { return nbt * 64; }                                   // 4 token waves x nbt x 16
 constexpr int dma_slab_bytes(int nbt) { return (k2BV + dma_tile_tokens(nbt)) * k2RowBytes; }  // 65536 at nbt = 4
-constexpr int dma_lds_bytes(int nbt) { return k2Slabs * dma_slab_bytes(nbt); }                // 131072 at nbt = 4
+constexpr int dma_lds_bytes(int nbt) { return dma_slabs(nbt) * dma_slab_bytes(nbt); }         // 131072 at nbt = 4
 
 __device__ __forceinline__ void dma16(const char* gptr, char* lds_wave_base) {
   __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(gptr),
@@ -552,6 +552,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   constexpr int k2BT = dma_tile_tokens(NBT);        // tokens per workgroup
   constexpr int kWaveTok = NBT * 16;                // tokens per wave
   constexpr int k2SlabBytes = dma_slab_bytes(NBT);
+  constexpr int k2Slabs = dma_slabs(NBT);           // with three, the barrier of a step no longer waits for the newest request
   constexpr int kBLoads = NBT;                      // DMA instructions per lane and slab for the hidden rows
   constexpr int k2DmaPerSlab = k2Loads + kBLoads;   // 8 at NBT = 4
 
@@ -615,13 +616,13 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   const int n_steps = (vt1 - vt0) * nk;
   const int64_t slab_rewind = (int64_t)(nk - 1) * k2RowBytes;
   int i_kt = 0, i_vt = vt0;  // slab the next `issue` will request
-  int issued = 0;            // slabs requested so far; request q lands in buffer q % 2
+  int issued = 0;            // slabs requested so far; request q lands in buffer q % k2Slabs
 
   // One of the eight DMA instructions of the next request (0-3: W rows; 4-7: hidden rows).
   auto issue_piece = [&](int piece) {
     // Past the last slab the request is repeated (same addresses, same buffer, identical bytes): it is
     // issued on every step so that the code has no branch and the wait counts stay static.
-    char* dst = smem + ((issued < n_steps ? issued : n_steps - 1) & (k2Slabs - 1)) * k2SlabBytes + wave * 1024;
+    char* dst = smem + ((unsigned)(issued < n_steps ? issued : n_steps - 1) % k2Slabs) * k2SlabBytes + wave * 1024;
     if (piece < k2Loads) dma16(pa[piece], dst + piece * 8192);
     else dma16(pb[piece - k2Loads], dst + k2BV * k2RowBytes + (piece - k2Loads) * 8192);
   };
@@ -643,28 +644,28 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   };
   // Fragments of one K = 32 sub-step of a slab: W blocks [i0, i0 + 4) or the four hidden blocks.
   auto read_a = [&](int slot, int ks, int i0, bf16x8 (&fa)[4]) {
-    const char* slab = smem + (slot & (k2Slabs - 1)) * k2SlabBytes;
+    const char* slab = smem + ((unsigned)slot % k2Slabs) * k2SlabBytes;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       fa[i] = *reinterpret_cast<const bf16x8*>(slab + (rdA ^ (ks * 64)) + (i0 + i) * 16 * k2RowBytes);
   };
   auto read_b = [&](int slot, int ks, bf16x8 (&fb)[k2NBT]) {
-    const char* slab = smem + (slot & (k2Slabs - 1)) * k2SlabBytes;
+    const char* slab = smem + ((unsigned)slot % k2Slabs) * k2SlabBytes;
 #pragma unroll
     for (int j = 0; j < k2NBT; ++j)
       fb[j] = *reinterpret_cast<const bf16x8*>(slab + (rdB ^ (ks * 64)) + j * 16 * k2RowBytes);
   };
 
-  for (int q = 0; q < 2; ++q) {
+  for (int q = 0; q < k2Slabs; ++q) {
 #pragma unroll
     for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
     issue_done();
   }
-  // slab 0 has landed (this wave's share): only the requests of slab 1 may still be in flight
-  if constexpr (k2DmaPerSlab == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-  else if constexpr (k2DmaPerSlab == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
-  __syncthreads();
+  // Slab 0 has landed (this wave's share): only the requests of the later slabs may still be in flight.
+  if constexpr (NBT == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");        // 1 slab x 8 requests
+  else if constexpr (NBT == 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");  // 2 slabs x 6
+  else asm volatile("s_waitcnt vmcnt(10)" ::: "memory");                          // 2 slabs x 5
+  __builtin_amdgcn_s_barrier();
 
   bf16x8 fa_lo[4], fa_hi[4], fb0[k2NBT], fb1[k2NBT];
   read_a(0, 0, 0, fa_lo);
@@ -709,7 +710,10 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     __builtin_amdgcn_sched_barrier(0);
     // This wave has read all it needs of slab `step` and its share of slab step+1 has landed; after
     // the (fence-less) barrier both hold for everyone.
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    // (With three buffers the requests of slab step+2 stay in flight across the barrier.)
+    if constexpr (NBT == 4) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    else if constexpr (NBT == 2) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     // Last quarter: first fragments of slab step+1 (after the last step a stale buffer, unused) and the
     // next request, which refills the buffer of slab `step`.  The DMA requests write LDS, so they keep
