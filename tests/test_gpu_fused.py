@@ -289,3 +289,22 @@ def test_fused_small_batch_kernel(dev, n, H, V, masked):
     assert (r.lp.cpu().numpy()[~m] == 0).all() and (r.argmax.cpu().numpy()[~m] == -1).all()
     plain = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 0.8)     # the variant without extras
     np.testing.assert_allclose(plain.lp.cpu().numpy(), want["lp"], atol=TOL, rtol=0)
+
+
+@pytest.mark.parametrize("n,H", [(10, 1024), (100, 1024), (50, 4096), (100, 2560), (300, 1024), (40, 72)])
+def test_fused_all_masked_and_single_valid_row(dev, n, H):
+    """Every sweep kernel (streaming with 1 / 4 / 8 token blocks, DMA with 64- / 128- / 256-token tiles, generic) with
+    no valid row at all - nothing may be read, every output is the masked value - and with exactly one."""
+    V = 5000
+    h, w, t = _inputs(dev, n, H, V, n + H, w_scale=0.05)
+    tt = torch.from_numpy(t).to(dev)
+    none = torch.zeros(n, dtype=torch.int32, device=dev)
+    r = tome_amd.fused_lmhead_logprobs(h, w, tt, 1.0, row_valid=none, want_entropy=True, want_argmax=True, want_lse=True)
+    assert (r.lp == 0).all() and (r.lse == 0).all() and (r.entropy == 0).all() and (r.argmax == -1).all()
+    one = none.clone()
+    one[n // 2] = 1
+    r = tome_amd.fused_lmhead_logprobs(h, w, tt, 1.0, row_valid=one)
+    want = oracle.lmhead_stats(bf16_bits_of(h[n // 2:n // 2 + 1]), bf16_bits_of(w), t[n // 2:n // 2 + 1], 1.0)
+    assert abs(r.lp[n // 2].item() - want["lp"][0]) < TOL and (r.lp[one == 0] == 0).all()
+    d = tome_amd.grpo_dual_logprobs(h, w, w, tt, 1.0, row_valid=one)
+    assert d.k3[n // 2].item() == 0.0 and (d.k3[one == 0] == 0).all()
