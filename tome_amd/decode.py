@@ -12,7 +12,7 @@ The model itself (KV cache, attention) is not part of this path: ``model_step(to
 """
 from __future__ import annotations
 
-from typing import Callable, List, Optional, Sequence
+from typing import Callable, List, Optional
 
 import numpy as np
 import torch
@@ -29,14 +29,21 @@ def _uniforms(source, step: int, rows: int, dev: torch.device, generator) -> Opt
     return torch.as_tensor(u, dtype=torch.float32, device=dev).reshape(rows)
 
 
-def _step(logits: torch.Tensor, temperature: float, top_k: int, uniforms, active: Optional[Sequence[bool]]):
-    """Sample every active row and fetch (token, lp) with one copy."""
-    dev = logits.device
-    rv = None if active is None else torch.tensor([1 if a else 0 for a in active], dtype=torch.int32, device=dev)
-    out = sample_tokens(logits, temperature, top_k, uniforms=uniforms if temperature > 0 else None, row_valid=rv)
+def _step(logits: torch.Tensor, temperature: float, top_k: int, uniforms, row_valid: Optional[torch.Tensor]):
+    """Sample every active row; returns the device token ids and, after ONE copy, the host (token, lp) arrays."""
+    out = sample_tokens(logits, temperature, top_k, uniforms=uniforms if temperature > 0 else None, row_valid=row_valid)
     host = torch.cat([out.token, out.lp.view(torch.int32)]).cpu().numpy()      # one sync, one copy
     n = out.token.numel()
-    return host[:n].astype(np.int64), host[n:].view(np.float32)
+    return out.token, host[:n].astype(np.int64), host[n:].view(np.float32)
+
+
+def _mask_to_device(active: np.ndarray, dev: torch.device) -> torch.Tensor:
+    return torch.from_numpy(active.astype(np.int32)).to(dev)
+
+
+def _results(toks: np.ndarray, lps: np.ndarray, lens: np.ndarray) -> List[dict]:
+    return [{"tokens": toks[i, :lens[i]].tolist(), "log_probs": [float(v) for v in lps[i, :lens[i]]]}
+            for i in range(toks.shape[0])]
 
 
 def rollout_decode(model_step: Callable[[torch.Tensor], torch.Tensor], last_logits: torch.Tensor, G: int,
@@ -53,33 +60,42 @@ def rollout_decode(model_step: Callable[[torch.Tensor], torch.Tensor], last_logi
     reaches ``max_tokens``.  Returns ``[{"tokens": [...], "log_probs": [...]}]`` in sequence order
     ``p_idx * G + g_idx`` (node.py:574).  ``uniform_source(step, rows)`` supplies the draws' uniforms
     (step 0 = first tokens); by default they come from ``torch.rand`` with ``generator``.
+
+    Per generated token the host does one device-to-host copy (tokens and log-probs of the batch) and array
+    bookkeeping; the next step's input ids are formed on the device from the sampled ids, and the row mask is
+    uploaded only when a sequence finishes.
     """
     dev = last_logits.device
     total = last_logits.shape[0] * G
     first = last_logits.repeat_interleave(G, dim=0)                            # same row, G independent draws
-    tok, lp = _step(first, temperature, top_k, _uniforms(uniform_source, 0, total, dev, generator), None)
-    results = [{"tokens": [int(tok[i])], "log_probs": [float(lp[i])]} for i in range(total)]    # node.py:574
-    active_tokens = [int(t) for t in tok]
-    finished = [False] * total                                                 # node.py:575: the first token is not checked
+    dev_tok, tok, lp = _step(first, temperature, top_k, _uniforms(uniform_source, 0, total, dev, generator), None)
+    width = max(int(max_tokens), 1)
+    toks = np.zeros((total, width), dtype=np.int64)
+    lps = np.zeros((total, width), dtype=np.float32)
+    lens = np.ones(total, dtype=np.int64)
+    toks[:, 0], lps[:, 0] = tok, lp                                            # node.py:574
+    finished = np.zeros(total, dtype=bool)                                     # node.py:575: the first token is not checked
+    rv_dev = None                                                              # None = every row active
+    eos_dev = torch.full((total,), int(eos_token_id), dtype=torch.int64, device=dev)
     for step in range(max_tokens - 1):                                         # node.py:578
-        if all(finished):
+        if finished.all():
             break
-        logits = model_step(torch.tensor(active_tokens, dtype=torch.int64, device=dev))
-        tok, lp = _step(logits, temperature, top_k, _uniforms(uniform_source, step + 1, total, dev, generator),
-                        [not f for f in finished])
-        new_active = []
-        for b in range(total):
-            if finished[b]:
-                new_active.append(eos_token_id)                                # node.py:593-595
-                continue
-            token = int(tok[b])
-            results[b]["tokens"].append(token)                                 # node.py:604-605
-            results[b]["log_probs"].append(float(lp[b]))
-            if token == eos_token_id or len(results[b]["tokens"]) >= max_tokens:
-                finished[b] = True                                             # node.py:607-608
-            new_active.append(token)
-        active_tokens = new_active
-    return results
+        inputs = dev_tok.to(torch.int64)
+        if rv_dev is not None:
+            inputs = torch.where(rv_dev != 0, inputs, eos_dev)                 # node.py:593-595
+        logits = model_step(inputs)
+        dev_tok, tok, lp = _step(logits, temperature, top_k, _uniforms(uniform_source, step + 1, total, dev, generator),
+                                 rv_dev)
+        act = ~finished
+        rows = np.nonzero(act)[0]
+        toks[rows, lens[rows]] = tok[rows]                                     # node.py:604-605
+        lps[rows, lens[rows]] = lp[rows]
+        lens[rows] += 1
+        newly = act & ((tok == eos_token_id) | (lens >= max_tokens))           # node.py:607-608
+        if newly.any():
+            finished |= newly
+            rv_dev = _mask_to_device(~finished, dev)
+    return _results(toks, lps, lens)
 
 
 def judge_decode(model_step: Callable[[torch.Tensor], torch.Tensor], first_logits: torch.Tensor,
@@ -95,24 +111,29 @@ def judge_decode(model_step: Callable[[torch.Tensor], torch.Tensor], first_logit
     """
     dev = first_logits.device
     B = first_logits.shape[0]
-    tok, lp = _step(first_logits, temperature, top_k, _uniforms(uniform_source, 0, B, dev, generator), None)
-    results = [{"tokens": [int(tok[i])], "log_probs": [float(lp[i])]} for i in range(B)]
-    active_tokens = [int(t) for t in tok]
-    active = [True] * B                                                        # node.py:344
+    dev_tok, tok, lp = _step(first_logits, temperature, top_k, _uniforms(uniform_source, 0, B, dev, generator), None)
+    width = max(int(max_tokens), 1)
+    toks = np.zeros((B, width), dtype=np.int64)
+    lps = np.zeros((B, width), dtype=np.float32)
+    lens = np.ones(B, dtype=np.int64)
+    toks[:, 0], lps[:, 0] = tok, lp
+    active = np.ones(B, dtype=bool)                                            # node.py:344
+    rv_dev = None
+    zero_dev = torch.zeros(B, dtype=torch.int64, device=dev)
     for step in range(max_tokens - 1):                                         # node.py:346
-        if not any(active):
+        if not active.any():
             break
-        inputs = [t if active[i] else 0 for i, t in enumerate(active_tokens)]  # node.py:350
-        logits = model_step(torch.tensor(inputs, dtype=torch.int64, device=dev))
-        tok, lp = _step(logits, temperature, top_k, _uniforms(uniform_source, step + 1, B, dev, generator), active)
-        for i in range(B):
-            if not active[i]:
-                continue
-            token = int(tok[i])
-            active_tokens[i] = token
-            if token == eos_token_id:
-                active[i] = False                                              # node.py:369-370
-            else:
-                results[i]["tokens"].append(token)                             # node.py:371-373
-                results[i]["log_probs"].append(float(lp[i]))
-    return results
+        inputs = dev_tok.to(torch.int64)
+        if rv_dev is not None:
+            inputs = torch.where(rv_dev != 0, inputs, zero_dev)                # node.py:350
+        logits = model_step(inputs)
+        dev_tok, tok, lp = _step(logits, temperature, top_k, _uniforms(uniform_source, step + 1, B, dev, generator), rv_dev)
+        ended = active & (tok == eos_token_id)                                 # node.py:369-370: EOS is not recorded
+        rows = np.nonzero(active & ~ended)[0]
+        toks[rows, lens[rows]] = tok[rows]                                     # node.py:371-373
+        lps[rows, lens[rows]] = lp[rows]
+        lens[rows] += 1
+        if ended.any():
+            active &= ~ended
+            rv_dev = _mask_to_device(active, dev)
+    return _results(toks, lps, lens)
