@@ -32,8 +32,13 @@ def _uniforms(source, step: int, rows: int, dev: torch.device, generator) -> Opt
 def _step(logits: torch.Tensor, temperature: float, top_k: int, uniforms, row_valid: Optional[torch.Tensor]):
     """Sample every active row; returns the device token ids and, after ONE copy, the host (token, lp) arrays."""
     out = sample_tokens(logits, temperature, top_k, uniforms=uniforms if temperature > 0 else None, row_valid=row_valid)
-    host = torch.cat([out.token, out.lp.view(torch.int32)]).cpu().numpy()      # one sync, one copy
     n = out.token.numel()
+    tok, lp = out.token.reshape(-1), out.lp.reshape(-1)
+    if lp.data_ptr() == tok.data_ptr() + 4 * n:        # the sampler's outputs sit back to back: no gather needed
+        both = torch.as_strided(tok, (2 * n,), (1,))
+    else:
+        both = torch.cat([tok, lp.view(torch.int32)])
+    host = both.cpu().numpy()                                                  # one sync, one copy
     return out.token, host[:n].astype(np.int64), host[n:].view(np.float32)
 
 

@@ -223,9 +223,8 @@ def sample_tokens(logits: torch.Tensor, temperature: float, top_k: int = 20, *, 
                 u = torch.as_tensor(uniforms, dtype=torch.float32, device=dev).reshape(-1).contiguous()
                 if u.numel() != rows:
                     raise ValueError(f"uniforms must have one value per row ({rows}), got {u.numel()}")
-        tok = torch.empty(rows, dtype=torch.int32, device=dev)
-        lp = torch.empty(rows, dtype=torch.float32, device=dev)
-        amax = torch.empty(rows, dtype=torch.int32, device=dev)
+        packed = torch.empty((3, rows), dtype=torch.int32, device=dev)   # token | lp bits | argmax: one allocation,
+        tok, lp, amax = packed[0], packed[1].view(torch.float32), packed[2]  # and (token, lp) leave in one copy
         tki = torch.empty((rows, top_k), dtype=torch.int32, device=dev) if want_topk else None
         tkl = torch.empty((rows, top_k), dtype=torch.float32, device=dev) if want_topk else None
         ws_bytes = lib.tome_row_sample_workspace(dtype, rows, V, int(top_k))
