@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define TOME_ABI_VERSION 1
+#define TOME_ABI_VERSION 2
 
 enum { TOME_F32 = 0, TOME_BF16 = 1 };
 
@@ -42,7 +42,8 @@ enum {
   TOME_E_WORKSPACE = -4,   /* workspace_bytes smaller than the *_workspace() query */
   TOME_E_TEMPERATURE = -5, /* temperature not finite or <= 0 */
   TOME_E_ALIGN = -6,       /* pointer or stride alignment the kernel needs is not met */
-  TOME_E_HIP = -7          /* a HIP runtime call failed; see tome_last_hip_error() */
+  TOME_E_HIP = -7,         /* a HIP runtime call failed; see tome_last_hip_error() */
+  TOME_E_SCRATCH = -8      /* tome_row_logprob_noalloc: the call needs more than the fixed scratch buffer */
 };
 
 int tome_abi_version(void);
@@ -65,6 +66,25 @@ int tome_row_logprob(const void* logits, int dtype, int64_t rows, int64_t V, int
                      const int32_t* targets, const int32_t* row_valid, float temperature,
                      float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
                      void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- Row kernel for callers that cannot allocate ------------------------------------
+ * No counterpart in the reference.  It exists for callers that cannot hand over a workspace
+ * because they cannot allocate one: code running under HIP graph capture, serving loops with
+ * a fixed memory plan, harnesses that forbid hipMalloc.  Same arguments, kernels and results
+ * as tome_row_logprob, minus the workspace: the per-(row, split) partials of small batches
+ * go to a fixed 64 KiB array inside the library's code object (one copy per GPU, held until
+ * the process ends).  The call allocates and frees nothing.  A call whose partials would not
+ * fit returns TOME_E_SCRATCH before any launch (with the library's split rule - fewer than
+ * 512 rows are split so that about 512 workgroups run - no shape needs more than 16 KiB).
+ * All calls on one GPU share the array: calls that overlap in time on the same GPU (different
+ * streams) race on it; calls on one stream, or on different GPUs, do not.  The first call on
+ * each GPU looks the array's address up (hipGetSymbolAddress); make that call outside any
+ * graph capture.
+ */
+int tome_row_logprob_noalloc(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                             const int32_t* targets, const int32_t* row_valid, float temperature,
+                             float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
+                             void* stream);
 
 /* ---- Decode-step sampler on the same logits pass -----------------------------------
  * Replaces, for a batch of decode rows, _sample_token(logits, temperature, top_k=20)

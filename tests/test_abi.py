@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(tome_amd.lib_path())
     for name in declared_functions():
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
-    assert tome_amd.load_library().tome_abi_version() == 1
+    assert tome_amd.load_library().tome_abi_version() == 2
 
 
 def test_header_cites_reference_for_each_entry_point():
@@ -41,7 +41,7 @@ def test_header_cites_reference_for_each_entry_point():
 def test_strerror_and_codes():
     lib = tome_amd.load_library()
     assert lib.tome_strerror(0) == b"ok"
-    for code in range(-7, 0):
+    for code in range(-8, 0):
         assert lib.tome_strerror(code) not in (b"ok", b"unknown error code")
     assert lib.tome_strerror(-99) == b"unknown error code"
 
@@ -74,6 +74,12 @@ def test_argument_checks_run_on_host():
     assert row(rows=0) == 0                        # empty batch is a no-op
     assert row(rows=64, V=151936, stride=151936) == -4   # split rows need a workspace
     assert row(logits=P + 1) == -6
+    na = lambda **k: lib.tome_row_logprob_noalloc(k.get("logits", P), k.get("dtype", 1), k.get("rows", 4), k.get("V", 64),
+                                                  k.get("stride", 64), k.get("targets", P), None, k.get("T", 1.0),
+                                                  k.get("lp", P), None, None, None, None)
+    assert na(dtype=7) == -2 and na(V=0) == -3 and na(stride=63) == -3 and na(T=0.0) == -5
+    assert na(logits=None) == -1 and na(targets=None) == -1 and na(lp=None) == -1 and na(rows=0) == 0
+    assert na(logits=P + 1) == -6
     fused = lambda **k: lib.tome_fused_lmhead_logprob(k.get("h", P), k.get("w", P), k.get("n", 8), k.get("H", 64),
                                                       k.get("V", 100), k.get("hs", 64), k.get("ws", 64), P, None,
                                                       k.get("T", 1.0), k.get("lp", P), None, None, None, None, 0, None)

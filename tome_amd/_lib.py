@@ -10,7 +10,7 @@ _LIB_PATH = os.path.join(_PKG_DIR, "libtome_logprob.so")
 _lib: ctypes.CDLL | None = None
 
 TOME_F32, TOME_BF16 = 0, 1
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # name -> (restype, argtypes); must list every function the header declares.
 SIGNATURES = {
@@ -20,6 +20,8 @@ SIGNATURES = {
     "tome_row_logprob_workspace": (c_size_t, [c_int64, c_int64]),
     "tome_row_logprob": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "tome_row_logprob_noalloc": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float,
+                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "tome_row_sample_workspace": (c_size_t, [c_int, c_int64, c_int64, c_int]),
     "tome_row_sample": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float, c_int,
                                 c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
@@ -93,6 +95,6 @@ def check(code: int) -> None:
     msg = lib.tome_strerror(code).decode()
     if code == -7:
         msg += f" [hipError_t {lib.tome_last_hip_error()}]"
-    if code in (-1, -2, -3, -5, -6):
+    if code in (-1, -2, -3, -5, -6, -8):
         raise ValueError(f"libtome_logprob: {msg} (code {code})")
     raise TomeError(code, msg)

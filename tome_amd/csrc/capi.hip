@@ -12,6 +12,10 @@ hipError_t row_logprob_launch(const void* logits, int dtype, int64_t rows, int64
                               float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
                               void* workspace, hipStream_t stream);
 int row_splits_for(int64_t rows, int64_t V, int vec);
+hipError_t row_logprob_noalloc_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                                      const int32_t* targets, const int32_t* row_valid, float temperature,
+                                      float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
+                                      bool* too_big, hipStream_t stream);
 hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t rows, int64_t V,
                                    int64_t in_stride, int64_t out_stride, float temperature,
                                    const float* row_lse, hipStream_t stream);
@@ -76,6 +80,7 @@ const char* tome_strerror(int code) {
     case TOME_E_TEMPERATURE: return "temperature must be finite and > 0";
     case TOME_E_ALIGN: return "pointer or stride not aligned as the kernel requires";
     case TOME_E_HIP: return "HIP runtime error (see tome_last_hip_error)";
+    case TOME_E_SCRATCH: return "the call needs more scratch than the allocation-free entry point's fixed buffer holds";
     default: return "unknown error code";
   }
 }
@@ -107,6 +112,25 @@ int tome_row_logprob(const void* logits, int dtype, int64_t rows, int64_t V, int
   return hip_result(tome::row_logprob_launch(logits, dtype, rows, V, row_stride, targets, row_valid, temperature,
                                              out_lp, out_lse, out_entropy, out_argmax, workspace,
                                              static_cast<hipStream_t>(stream)));
+}
+
+int tome_row_logprob_noalloc(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                             const int32_t* targets, const int32_t* row_valid, float temperature, float* out_lp,
+                             float* out_lse, float* out_entropy, int32_t* out_argmax, void* stream) {
+  if (dtype != TOME_F32 && dtype != TOME_BF16) return TOME_E_DTYPE;
+  if (bad_matrix(rows, V, row_stride)) return TOME_E_SHAPE;
+  if (bad_temperature(temperature)) return TOME_E_TEMPERATURE;
+  if (rows == 0) return TOME_OK;
+  if (!logits) return TOME_E_NULL;
+  if (out_lp && !targets) return TOME_E_NULL;
+  if (!out_lp && !out_lse && !out_entropy && !out_argmax) return TOME_E_NULL;
+  if (reinterpret_cast<uintptr_t>(logits) % (dtype == TOME_F32 ? 4 : 2) != 0) return TOME_E_ALIGN;
+  bool too_big = false;
+  const hipError_t e = tome::row_logprob_noalloc_launch(logits, dtype, rows, V, row_stride, targets, row_valid,
+                                                        temperature, out_lp, out_lse, out_entropy, out_argmax,
+                                                        &too_big, static_cast<hipStream_t>(stream));
+  if (too_big) return TOME_E_SCRATCH;
+  return hip_result(e);
 }
 
 size_t tome_row_sample_workspace(int dtype, int64_t rows, int64_t V, int top_k) {

@@ -13,6 +13,8 @@
 // results do not depend on scheduling).
 #include "row_common.hpp"
 
+#include <mutex>
+
 namespace tome {
 
 struct RowPartial {  // one per (row, split) in the workspace
@@ -244,6 +246,65 @@ hipError_t row_logprob_launch(const void* logits, int dtype, int64_t rows, int64
   }
   return vector_ok ? dispatch_flags<uint16_t, true>(a, rows, stream)
                    : dispatch_flags<uint16_t, false>(a, rows, stream);
+}
+
+// ---- allocation-free variant ---------------------------------------------------------------------
+// The per-(row, split) partials of a split launch normally live in a caller-provided workspace.  For
+// callers that cannot allocate one (code under graph capture, serving loops with a fixed memory plan)
+// the same launches can use this array, which is part of the code object: every GPU the library runs on
+// holds its own copy from the first launch until the process ends.  In host code the array's name is
+// only a handle for hipGetSymbolAddress; kernels are given the address it returns for the current
+// device.  Nothing in it has to start at zero: the combine kernel reads exactly the partials that the
+// main kernel of the same call wrote.  All calls on one GPU share the array, so two calls that overlap
+// in time on one GPU (different streams) race on it.
+constexpr size_t kRowScratchBytes = 64 * 1024;
+static __device__ __align__(256) unsigned char scratch[kRowScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch`, per device ordinal
+static std::mutex g_scratch_mutex;
+
+size_t row_scratch_capacity() { return kRowScratchBytes; }
+
+// Address of this device's copy of the scratch array; resolved once per device, with that device current.
+static hipError_t row_scratch_for_current_device(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return hipSuccess;
+}
+
+// Bytes of partials a call with these shapes writes (0 when every row is one workgroup).
+size_t row_partials_bytes(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride) {
+  const int vec = 16 / (dtype == 0 ? 4 : 2);
+  const bool vector_ok = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && (row_stride % vec == 0);
+  const int splits = row_splits_for(rows, V, vector_ok ? vec : 1);
+  return splits <= 1 ? 0 : (size_t)rows * (size_t)splits * sizeof(RowPartial);
+}
+
+// row_logprob_launch with the partials in the library's own scratch array.  `too_big` is set (and nothing
+// launched) when the call would need more than the array holds.
+hipError_t row_logprob_noalloc_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                                      const int32_t* targets, const int32_t* row_valid, float temperature,
+                                      float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
+                                      bool* too_big, hipStream_t stream) {
+  *too_big = row_partials_bytes(logits, dtype, rows, V, row_stride) > kRowScratchBytes;
+  if (*too_big) return hipSuccess;
+  void* ptr = nullptr;
+  const hipError_t e = row_scratch_for_current_device(&ptr);
+  if (e != hipSuccess) return e;
+  return row_logprob_launch(logits, dtype, rows, V, row_stride, targets, row_valid, temperature, out_lp, out_lse,
+                            out_entropy, out_argmax, ptr, stream);
 }
 
 }  // namespace tome
