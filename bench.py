@@ -1,14 +1,21 @@
 #!/usr/bin/env python3
 """Benchmark of the token-log-prob path on one MI355X.
 
-A step is one pass of the hot path over one batch of synthetic input that is already
-resident in HBM.  The headline workload is benchmark configuration 2 (the Qwen3-0.6B GRPO
-ref-logprob shape: bf16 logits [8 x 512, 151936] with a padding mask); the same JSON line
-also carries the unmasked variant, the fused lm_head + log-softmax kernel at configuration 3
-(4096 tokens) and at a decode-step batch (64 tokens), one decode step's sampler, and the LoRA
-merge of one UpdateWeights request.
+A step is one pass of the hot path over one batch of synthetic input that is already resident in
+HBM.  The headline workload is benchmark configuration 2 (the Qwen3-0.6B GRPO ref-logprob shape:
+bf16 logits [8 x 512, 151936] with a padding mask).  The same JSON line carries one object per
+further workload: configuration 2 without its mask, configuration 1 (64 x 151936 fp32, the
+CPU-comparison shape), the fused lm_head + log-softmax kernel at configurations 3, 4 and 5, the same
+entry at decode-step and small-batch sizes, one decode step's sampler, and the LoRA merge of one
+UpdateWeights request.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only row|fused|small|decode|lora]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only LEG[,LEG...]]
+
+Every leg does W untimed warm-up steps, then an untimed settle phase (launches until the GPU has been
+busy for SETTLE_MS, so that clocks have left their idle state; the count is reported as
+`settle_launches`), then times EXACTLY K back-to-back steps between two HIP events on the launch
+stream (`ms_per_step`, the mean), and finally repeats K steps with an event between launches for the
+median of the per-launch times (`median_ms`, `min_ms`; this second pass does not feed `ms_per_step`).
 
 Prints ONE JSON line on stdout.  Everything else goes to stderr.
 """
@@ -25,21 +32,35 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 V = 151936
-HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
-# HBM-side bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE counter passes, each scaled by the same
-# counter's reading for a plain 2^30-byte copy (profiles/hbm_traffic_counters.txt).  The masked figure
-# belongs to the seeded lengths of make_config2 (2356 valid rows).
-TRAFFIC_ROW_MASKED = 716.4e6 + 0.13e6
-TRAFFIC_ROW_ALL = 1245.0e6 + 0.13e6
-TRAFFIC_FUSED_CFG3 = 1847e6 + 6.8e6
-TRAFFIC_DECODE_64 = 39.2e6 + 0.30e6 + 0.23e6   # sampler: main-kernel fetch, combine fetch, partials written
-TRAFFIC_FUSED_SMALL_64 = 326.0e6 + 0.52e6      # sweep kernel: fetch + partials written (profiles/fused_lmhead_small_kernel_decode_64tokens.txt)
-TRAFFIC_LORA_06B = 812.1e6 + 763.4e6            # merge kernel: fetch + write (profiles/lora_merge_kernel_qwen3_0.6b_update.txt)
+SETTLE_MS = 60.0                # untimed GPU-busy time in front of every timed region (default of --settle-ms)
+SETTLE = {"ms": SETTLE_MS}
+SETTLE_MAX_LAUNCHES = 2000
+LEGS = ["row", "config1", "ceiling", "fused", "config4", "config5", "small", "midsize", "decode", "lora"]
+SUSTAINED = {"tflops": None}    # bf16 MFMA rate of the probe loop on random operands, measured by the `ceiling` leg
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def load_counters():
+    """HBM-side traffic per launch and the sustained MFMA rate, as measured with rocprofv3 and recorded
+    beside the summaries they come from (profiles/counters.json).  Missing entries read as None."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "counters.json")) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {}
+
+
+COUNTERS = load_counters()
+
+
+def traffic_of(key):
+    e = COUNTERS.get("traffic", {}).get(key)
+    return None if e is None else float(e["fetch_bytes"]) + float(e["write_bytes"])
 
 
 def make_config2(dev, seed=1234):
@@ -63,12 +84,27 @@ def make_config2(dev, seed=1234):
 
 
 def time_steps(fn, steps, warmup):
-    """Average milliseconds per step over `steps` back-to-back launches, by HIP events recorded on
-    the stream the kernels run on (torch's current stream, which the library launches into)."""
+    """Warm-up, settle, timed region, per-launch pass (see the module docstring).  Times in milliseconds by
+    HIP events recorded on the stream the kernels run on (torch's current stream, which the library
+    launches into)."""
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    # settle: untimed launches until the GPU has been busy for SETTLE_MS
+    settle, busy, batch = 0, 0.0, 1
+    while busy < SETTLE["ms"] and settle < SETTLE_MAX_LAUNCHES:
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        if settle:   # size the next batch from the time per launch seen so far
+            batch = int(min(max(1.0, (SETTLE["ms"] - busy) / (busy / settle)) + 1, 200, SETTLE_MAX_LAUNCHES - settle))
+        a.record()
+        for _ in range(batch):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        busy += a.elapsed_time(b)
+        settle += batch
+    # the timed region: exactly `steps` launches between two events
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     start.record()
@@ -77,9 +113,41 @@ def time_steps(fn, steps, warmup):
     stop.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return start.elapsed_time(stop) / steps, wall_ms
+    mean_ms = start.elapsed_time(stop) / steps
+    # per-launch times: a second pass with an event between launches
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    ev[0].record()
+    for i in range(steps):
+        fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(steps))
+    return {"ms": mean_ms, "wall_ms": wall_ms, "median_ms": per[len(per) // 2], "min_ms": per[0],
+            "settle_launches": settle}
 
 
+def timing_fields(t):
+    return {"ms_per_step": t["ms"], "median_ms": t["median_ms"], "min_ms": t["min_ms"],
+            "settle_launches": t["settle_launches"]}
+
+
+def hbm_roofline(nbytes, ms, traffic, kernel):
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+            "traffic": traffic, "kernel": kernel, "bytes_per_launch": nbytes}
+
+
+def mfma_roofline(flop, ms, traffic, kernel):
+    tf = flop / (ms * 1e-3) / 1e12
+    r = {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+         "frac": tf / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic, "kernel": kernel, "flop_per_launch": flop}
+    if SUSTAINED["tflops"]:   # what the bare LDS -> MFMA loop reaches on random bf16 operands, same run (`ceiling` leg)
+        r["sustained_peak"] = SUSTAINED["tflops"]
+        r["frac_of_sustained"] = tf / SUSTAINED["tflops"]
+    return r
+
+
+# ---- row kernel: configuration 2 (headline) and configuration 1 -----------------------------------------
 def bench_row(dev, steps, warmup, variant="both"):
     import torch
     import tome_amd
@@ -102,39 +170,74 @@ def bench_row(dev, steps, warmup, variant="both"):
                                         valid.data_ptr() if mask else None, 1.0, lp.data_ptr(), None, None, None,
                                         ws.data_ptr(), ws_bytes, stream))
 
-    # correctness gate on what is being timed: spike rows must score the closed form's ballpark
+    # correctness gate on what is being timed: log-probs are finite and <= 0, masked rows are zero
     step(True)
     torch.cuda.synchronize()
     got = lp.clone()
     assert torch.isfinite(got).all() and (got <= 1e-5).all()
     assert (got[valid == 0] == 0).all()
 
-    ms_mask, wall_mask = time_steps(lambda: step(True), steps, warmup) if variant in ("both", "mask") else (float("nan"),) * 2
-    ms_all, wall_all = time_steps(lambda: step(False), steps, warmup) if variant in ("both", "all") else (float("nan"),) * 2
-    bytes_mask = n_valid * V * 2
-    bytes_all = rows * V * 2
-    out = {
-        "n_valid": n_valid, "rows": rows,
-        "ms_mask": ms_mask, "ms_all": ms_all, "wall_ms_mask": wall_mask,
-        "gbs_mask": bytes_mask / (ms_mask * 1e-3) / 1e9, "gbs_all": bytes_all / (ms_all * 1e-3) / 1e9,
-        "bytes_mask": bytes_mask, "bytes_all": bytes_all,
-    }
+    out = {"n_valid": n_valid, "rows": rows, "bytes_mask": n_valid * V * 2, "bytes_all": rows * V * 2}
+    if variant in ("both", "mask"):
+        out["mask"] = time_steps(lambda: step(True), steps, warmup)
+    if variant in ("both", "all"):
+        out["all"] = time_steps(lambda: step(False), steps, warmup)
     del logits, flat
     torch.cuda.empty_cache()
     return out
 
 
-def bench_fused(dev, steps, warmup, n=4096, H=1024):
-    """Fused lm_head + log-softmax on [n, H] x [V, H]: config 3 by default; n = 64 is the decode-step batch,
-    where W is streamed once and the kernel is HBM-bound."""
+def bench_config1(dev, steps, warmup):
+    """Configuration 1: 64 rows x 151936 fp32 logits ~ N(0, 2^2), uniform targets - the shape of the reference's
+    CPU path (mlx-impl/node.py:400-404).  38.9 MB per launch would sit in the 256 MB last-level cache, so the
+    launches rotate through 16 buffers (622 MB) and every row comes from HBM."""
     import torch
     import tome_amd
     from tome_amd import _lib
     lib = tome_amd.load_library()
-    g = torch.Generator(device=dev).manual_seed(4321)
+    rows, nbuf = 64, 16
+    g = torch.Generator(device=dev).manual_seed(11)
+    xs = [torch.randn((rows, V), device=dev, generator=g) * 2.0 for _ in range(nbuf)]
+    t = torch.randint(0, V, (rows,), device=dev, generator=g).to(torch.int32)
+    lp = torch.empty(rows, dtype=torch.float32, device=dev)
+    ws_bytes = lib.tome_row_logprob_workspace(rows, V)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    i = [0]
+
+    def step():
+        x = xs[i[0] % nbuf]
+        i[0] += 1
+        _lib.check(lib.tome_row_logprob(x.data_ptr(), 0, rows, V, V, t.data_ptr(), None, 1.0, lp.data_ptr(), None, None,
+                                        None, ws.data_ptr(), ws_bytes, stream))
+    step()
+    torch.cuda.synchronize()
+    want = torch.log_softmax(xs[0].double(), dim=-1)[torch.arange(rows, device=dev), t.long()]
+    assert (lp.double() - want).abs().max().item() < 1e-4        # gate on what is timed (fp32 logits: 1e-4 abs)
+    tm = time_steps(step, steps, warmup)
+    tm.update({"rows": rows, "bytes": rows * V * 4})
+    return tm
+
+
+# ---- fused lm_head + log-softmax ---------------------------------------------------------------------
+def bench_fused(dev, steps, warmup, n=4096, H=1024, temperature=1.0, lengths=None, seed=4321):
+    """Fused lm_head + log-softmax on [n, H] x [V, H]: config 3 by default.  `lengths` = (sequences, L, lo, hi)
+    gives the padding mask of config 4 (per-sequence valid prefixes, lengths uniform in [lo, hi])."""
+    import torch
+    import tome_amd
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    g = torch.Generator(device=dev).manual_seed(seed)
     hidden = torch.randn((n, H), device=dev, generator=g).to(torch.bfloat16)
     weight = (torch.randn((V, H), device=dev, generator=g) * 0.02).to(torch.bfloat16)
     targets = torch.randint(0, V, (n,), device=dev, generator=g).to(torch.int32)
+    valid, n_valid = None, n
+    if lengths is not None:
+        S, L, lo, hi = lengths
+        assert S * L == n
+        lens = torch.randint(lo, hi + 1, (S,), device=dev, generator=g)
+        valid = (torch.arange(L, device=dev)[None, :] < lens[:, None]).to(torch.int32).reshape(-1).contiguous()
+        n_valid = int(valid.sum().item())
     lp = torch.empty(n, dtype=torch.float32, device=dev)
     ws_bytes = lib.tome_fused_lmhead_logprob_workspace(n, H, V)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
@@ -142,14 +245,92 @@ def bench_fused(dev, steps, warmup, n=4096, H=1024):
 
     def step():
         _lib.check(lib.tome_fused_lmhead_logprob(hidden.data_ptr(), weight.data_ptr(), n, H, V, H, H,
-                                                 targets.data_ptr(), None, 1.0, lp.data_ptr(), None, None, None,
+                                                 targets.data_ptr(), valid.data_ptr() if valid is not None else None,
+                                                 temperature, lp.data_ptr(), None, None, None,
                                                  ws.data_ptr(), ws_bytes, stream))
     step()
     torch.cuda.synchronize()
     assert torch.isfinite(lp).all() and (lp <= 1e-5).all()
-    ms, wall = time_steps(step, steps, warmup)
-    flop = 2.0 * n * H * V
-    return {"tokens": n, "H": H, "ms": ms, "wall_ms": wall, "tflops": flop / (ms * 1e-3) / 1e12, "flop": flop}
+    # gate on what is timed: 64 valid rows against a plain fp32 matmul + log_softmax
+    idx = (torch.arange(n, device=dev) if valid is None else torch.nonzero(valid).view(-1))[:: max(1, n_valid // 64)][:64]
+    ref = torch.log_softmax((hidden[idx].float() @ weight.float().T) / temperature, dim=-1)
+    ref = ref[torch.arange(idx.numel(), device=dev), targets[idx].long()]
+    assert (lp[idx] - ref).abs().max().item() < 2e-3
+    del ref
+    tm = time_steps(step, steps, warmup)
+    tm.update({"tokens": n, "valid": n_valid, "H": H, "flop": 2.0 * n_valid * H * V,
+               "bytes": V * H * 2 + n_valid * H * 2})
+    return tm
+
+
+def bench_dual(dev, steps, warmup, n=32 * 2048, H=4096):
+    """Configuration 5: GRPO policy + reference dual pass, two weight sets [V, 4096] (ref = policy + N(0, 0.002^2)),
+    hidden [32 x 2048, 4096]; outputs lp, ref_lp, k3 and entropy per token."""
+    import torch
+    import tome_amd
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    g = torch.Generator(device=dev).manual_seed(555)
+    hidden = torch.empty((n, H), device=dev, dtype=torch.bfloat16)
+    for i in range(0, n, 8192):
+        hidden[i:i + 8192] = torch.randn((min(8192, n - i), H), device=dev, generator=g).to(torch.bfloat16)
+    w_pol = torch.empty((V, H), device=dev, dtype=torch.bfloat16)
+    w_ref = torch.empty((V, H), device=dev, dtype=torch.bfloat16)
+    for i in range(0, V, 16384):
+        m = min(16384, V - i)
+        wp = (torch.randn((m, H), device=dev, generator=g) * 0.02).to(torch.bfloat16)
+        w_pol[i:i + m] = wp
+        w_ref[i:i + m] = (wp.float() + torch.randn((m, H), device=dev, generator=g) * 0.002).to(torch.bfloat16)
+    targets = torch.randint(0, V, (n,), device=dev, generator=g).to(torch.int32)
+    outs = [torch.empty(n, dtype=torch.float32, device=dev) for _ in range(4)]
+    ws_bytes = lib.tome_grpo_dual_workspace(n, H, V)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def step():
+        _lib.check(lib.tome_grpo_dual(hidden.data_ptr(), w_pol.data_ptr(), w_ref.data_ptr(), n, H, V, H, H,
+                                      targets.data_ptr(), None, 1.0, outs[0].data_ptr(), outs[1].data_ptr(),
+                                      outs[2].data_ptr(), outs[3].data_ptr(), ws.data_ptr(), ws_bytes, stream))
+    step()
+    torch.cuda.synchronize()
+    lp, ref_lp, k3, ent = outs
+    assert torch.isfinite(lp).all() and (lp <= 1e-5).all() and (k3 >= 0).all() and (ent > 0).all()
+    idx = torch.arange(0, n, n // 32, device=dev)[:32]
+    for w, got in ((w_pol, lp), (w_ref, ref_lp)):       # gate: 32 rows of each weight set against fp32 torch
+        ref = torch.log_softmax(hidden[idx].float() @ w.float().T, dim=-1)[torch.arange(32, device=dev), targets[idx].long()]
+        assert (got[idx] - ref).abs().max().item() < 2e-3
+    tm = time_steps(step, steps, warmup)
+    tm.update({"tokens": n, "H": H, "flop": 2.0 * 2.0 * n * H * V, "bytes": 2 * V * H * 2 + n * H * 2})
+    return tm
+
+
+def bench_ceiling(dev, steps, warmup, operands="random"):
+    """The fused kernel's LDS -> MFMA inner loop alone (tome_probe_mfma_ceiling): one workgroup per CU, operands
+    copied into LDS once, no global loads, barriers or epilogue in the loop.  `random`: W rows ~N(0, 0.02^2) and
+    token rows ~N(0, 1) as in config 3; `constant`: every operand 1.0."""
+    import torch
+    import tome_amd
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    g = torch.Generator(device=dev).manual_seed(31)
+    if operands == "random":
+        ops = torch.cat([torch.randn(256 * 64, device=dev, generator=g) * 0.02, torch.randn(256 * 64, device=dev, generator=g)])
+    else:
+        ops = torch.ones(512 * 64, device=dev)
+    ops = ops.to(torch.bfloat16).contiguous()
+    n_wg = torch.cuda.get_device_properties(dev).multi_processor_count
+    k_steps = 1024                                      # 64-wide K slabs per launch: about 1 ms
+    sink = torch.empty(n_wg * 512, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def step():
+        _lib.check(lib.tome_probe_mfma_ceiling(ops.data_ptr(), n_wg, k_steps, sink.data_ptr(), stream))
+    step()
+    torch.cuda.synchronize()
+    assert torch.isfinite(sink).all()
+    tm = time_steps(step, steps, warmup)
+    tm.update({"flop": float(n_wg) * k_steps * 2 * 256 * 256 * 64, "workgroups": n_wg, "k_steps": k_steps})
+    return tm
 
 
 def bench_decode(dev, steps, warmup):
@@ -178,8 +359,9 @@ def bench_decode(dev, steps, warmup):
     step()
     torch.cuda.synchronize()
     assert (tok >= 0).all() and (tok < V).all() and torch.isfinite(lp).all()
-    ms, wall = time_steps(step, steps, warmup)
-    return {"rows": rows, "top_k": k, "ms": ms, "bytes": rows * V * 4}
+    tm = time_steps(step, steps, warmup)
+    tm.update({"rows": rows, "top_k": k, "bytes": rows * V * 4})
+    return tm
 
 
 def bench_lora(dev, steps, warmup):
@@ -219,43 +401,56 @@ def bench_lora(dev, steps, warmup):
     base, out, a, b = keep[:4]                      # gate on what is timed: the first merge against fp32 torch
     want = base.float() + 2.5 * (b.float() @ a.float())
     assert (out.float() - want).abs().max().item() <= 2.0 ** -8 * want.abs().max().item() + 1e-3
-    ms, wall = time_steps(step, steps, warmup)
-    return {"ms": ms, "wall_ms": wall, "bytes": n_bytes, "jobs": len(jobs), "rank": rank}
+    tm = time_steps(step, steps, warmup)
+    tm.update({"bytes": n_bytes, "jobs": len(jobs), "rank": rank})
+    return tm
 
 
-def cpu_baseline(sample_rows=1024, budget_s=12.0):
-    """NumPy fp32 restatement of local_compute_logprobs (mlx-impl/node.py:400-404) on a bounded
-    sample of the config-2 workload: `sample_rows` rows of bf16 logits, upcast included."""
+# ---- CPU baseline -------------------------------------------------------------------------------------
+def cpu_baseline(budget_s=10.0):
+    """The reference's CPU path, local_compute_logprobs (mlx-impl/node.py:400-404), on configuration 1 (64 rows x
+    151936 fp32 logits ~ N(0, 2^2), uniform targets): the oracle's NumPy fp32 restatement (one core), the same
+    arithmetic with torch's CPU operators (its thread count stated) and in scalar C with OpenMP over rows."""
     import numpy as np
     import oracle
+    rows = 64
     rng = np.random.default_rng(99)
-    x = (rng.standard_normal((sample_rows, V)) * 3.0).astype(np.float32)
-    t = rng.integers(0, V, size=sample_rows).astype(np.int32)
-    x[np.arange(sample_rows), t] += 15.0
-    bits = oracle.bf16_round(x)
-    oracle.local_compute_logprobs_f32(bits[:8], t[:8], 1.0)   # warm-up
-    times = []
-    t_end = time.perf_counter() + budget_s
-    while time.perf_counter() < t_end and len(times) < 40:
-        t0 = time.perf_counter()
-        oracle.local_compute_logprobs_f32(bits, t, 1.0)
-        times.append(time.perf_counter() - t0)
-    med = sorted(times)[len(times) // 2]
-    out = {"value": sample_rows / med, "unit": "token-logprobs/s", "cores": 1, "kind": "port",
-           "sample": f"{sample_rows} rows x {V} bf16 logits (config-2 distribution), NumPy fp32 restatement of "
-                     f"node.py:400-404, median of {len(times)} passes"}
-    # multi-core figure: the same arithmetic in scalar C with OpenMP over rows
-    try:
+    x = (rng.standard_normal((rows, V)) * 2.0).astype(np.float32)
+    t = rng.integers(0, V, size=rows).astype(np.int32)
+
+    def median_time(fn, budget, cap=200):
+        fn()
+        times = []
+        t_end = time.perf_counter() + budget
+        while time.perf_counter() < t_end and len(times) < cap:
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        return sorted(times)[len(times) // 2], len(times)
+
+    med, n = median_time(lambda: oracle.local_compute_logprobs_f32(x, t, 1.0), budget_s)
+    out = {"value": rows / med, "unit": "token-logprobs/s", "cores": 1, "kind": "port",
+           "sample": f"config 1: {rows} rows x {V} fp32 logits, NumPy fp32 restatement of node.py:400-404 "
+                     f"(oracle.local_compute_logprobs_f32), median of {n} passes"}
+    try:   # the same expression on torch's CPU operators: the multi-threaded library figure
+        import torch
+        xt, tt = torch.from_numpy(x), torch.from_numpy(t.astype(np.int64))
+
+        def torch_pass():
+            z = xt / 1.0
+            return torch.take_along_dim(z, tt[:, None], dim=-1)[:, 0] - torch.logsumexp(z, dim=-1)
+        med_t, n_t = median_time(torch_pass, budget_s / 2)
+        out["torch_cpu"] = {"value": rows / med_t, "cores": torch.get_num_threads(), "kind": "port",
+                            "sample": f"same rows, torch CPU operators (x / T, logsumexp, take_along_dim), "
+                                      f"torch.get_num_threads() = {torch.get_num_threads()}, median of {n_t} passes"}
+    except Exception as e:
+        log("cpu torch baseline skipped:", e)
+    try:   # scalar C with OpenMP over rows
         from oracle import cport
         threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-        cport.local_compute_logprobs_c(bits[:8], t[:8], 1.0)
-        ts = []
-        for _ in range(10):
-            t0 = time.perf_counter()
-            cport.local_compute_logprobs_c(bits, t, 1.0)
-            ts.append(time.perf_counter() - t0)
-        out["multicore"] = {"value": sample_rows / min(ts), "cores": threads, "kind": "port",
-                            "sample": "same rows, scalar C + OpenMP restatement (oracle/metal_logsoftmax.c)"}
+        med_c, n_c = median_time(lambda: cport.local_compute_logprobs_c(x, t, 1.0), budget_s / 4)
+        out["multicore"] = {"value": rows / med_c, "cores": threads, "kind": "port",
+                            "sample": f"same rows, scalar C + OpenMP restatement (oracle/metal_logsoftmax.c), median of {n_c} passes"}
     except Exception as e:  # the C port is optional for the baseline
         log("cpu multicore baseline skipped:", e)
     return out
@@ -264,10 +459,12 @@ def cpu_baseline(sample_rows=1024, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
+                    help="untimed GPU-busy time in front of every timed region (counter runs pass 0)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["row", "fused", "small", "decode", "lora"], default=None)
+    ap.add_argument("--only", default=None, help="comma-separated subset of: " + ", ".join(LEGS))
     ap.add_argument("--row-variant", choices=["both", "mask", "all"], default="both",
                     help="time config 2 with its padding mask, without it, or both (profiling runs pick one)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -277,6 +474,11 @@ def main():
         log("bench.py: this path is measured on ONE GPU (rows are independent; more GPUs would each run "
             "this same kernel on their own share of the tokens). --gpus must be 1.")
         sys.exit(2)
+    only = LEGS if args.only is None else [s for s in args.only.split(",") if s]
+    for s in only:
+        if s not in LEGS:
+            log(f"bench.py: unknown leg {s!r}; choose from {LEGS}")
+            sys.exit(2)
 
     import torch
     import tome_amd
@@ -295,102 +497,148 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    row = bench_row(dev, args.steps, args.warmup, args.row_variant) if args.only in (None, "row") else None
-    # the fused step is ~10x longer than a row step: half the launches keep the run short; the clocks
-    # still settle (a few tens of milliseconds of back-to-back launches are needed for that)
-    fused = bench_fused(dev, max(5, args.steps // 2), max(2, args.warmup // 2)) if args.only in (None, "fused") else None
-    small = bench_fused(dev, args.steps, args.warmup, n=64) if args.only in (None, "small") else None
-    decode = bench_decode(dev, args.steps, args.warmup) if args.only in (None, "decode") else None
-    lora = bench_lora(dev, max(5, args.steps // 4), max(2, args.warmup // 4)) if args.only in (None, "lora") else None
+    K, W = args.steps, args.warmup
+    SETTLE["ms"] = args.settle_ms
+    legs = {}   # name -> JSON object; the first one present also becomes the top-level line
+
+    def done(name):
+        log(f"{name}: {legs[name]['ms_per_step'] * 1e3:.1f} us/step (median {legs[name]['median_ms'] * 1e3:.1f}), "
+            f"roofline {legs[name]['roofline']['frac']:.3f}")
+        torch.cuda.empty_cache()
+
+    if "row" in only:
+        row = bench_row(dev, K, W, args.row_variant)
+        if "mask" in row:
+            t = row["mask"]
+            legs["headline"] = {
+                "value": row["n_valid"] / (t["ms"] * 1e-3), "unit": "token-logprobs/s", **timing_fields(t),
+                "dtype": "f32", "input_dtype": "bf16",
+                "config": {"workload": "config 2: row log-softmax + target gather, bf16 logits [8x512, 151936], "
+                                       "padding mask lengths~U[64,512], fp32 out",
+                           "rows": row["rows"], "valid_rows": row["n_valid"], "vocab": V, "temperature": 1.0},
+                "roofline": hbm_roofline(row["bytes_mask"], t["ms"], traffic_of("row_logprob_config2_masked"),
+                                         "row_logprob_kernel<bf16>")}
+            done("headline")
+        if "all" in row:
+            t = row["all"]
+            legs["all_rows"] = {
+                "value": row["rows"] / (t["ms"] * 1e-3), "unit": "token-logprobs/s", **timing_fields(t),
+                "dtype": "f32", "input_dtype": "bf16",
+                "config": {"workload": "config 2 without the padding mask: all 4096 rows of bf16 logits [4096, 151936] read",
+                           "rows": row["rows"], "vocab": V, "temperature": 1.0},
+                "roofline": hbm_roofline(row["bytes_all"], t["ms"], traffic_of("row_logprob_config2_all_rows"),
+                                         "row_logprob_kernel<bf16>")}
+            done("all_rows")
+    if "config1" in only:
+        t = bench_config1(dev, K, W)
+        legs["config1_row"] = {
+            "value": t["rows"] / (t["ms"] * 1e-3), "unit": "token-logprobs/s", **timing_fields(t), "dtype": "f32",
+            "config": {"workload": "config 1: row log-softmax + target gather, fp32 logits [64, 151936] ~N(0,2^2), "
+                                   "uniform targets; 16 rotating input buffers (rows come from HBM)",
+                       "rows": t["rows"], "vocab": V, "temperature": 1.0},
+            "roofline": hbm_roofline(t["bytes"], t["ms"], traffic_of("row_logprob_config1"),
+                                     "row_logprob_kernel<f32> (8 workgroups per row) + row_combine_kernel")}
+        done("config1_row")
+    if "ceiling" in only:
+        t = bench_ceiling(dev, K, W, "random")
+        c = bench_ceiling(dev, K, W, "constant")
+        SUSTAINED["tflops"] = t["flop"] / (t["ms"] * 1e-3) / 1e12
+        legs["mfma_ceiling"] = {
+            "value": SUSTAINED["tflops"], "unit": "TFLOP/s", **timing_fields(t), "dtype": "bf16 x bf16 -> f32",
+            "config": {"workload": "bare LDS -> MFMA loop of the fused kernel (256x256 workgroup tile, v_mfma_f32_16x16x32_bf16, "
+                                   "one workgroup per CU, operands resident in LDS): random operands as in config 3",
+                       "workgroups": t["workgroups"], "k_slabs_per_launch": t["k_steps"],
+                       "constant_operands_tflops": c["flop"] / (c["ms"] * 1e-3) / 1e12},
+            "roofline": {"bound": "mfma", "achieved": SUSTAINED["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": SUSTAINED["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "kernel": "mfma_ceiling_kernel",
+                         "flop_per_launch": t["flop"]}}
+        done("mfma_ceiling")
+    if "fused" in only:
+        t = bench_fused(dev, K, W)
+        legs["fused_lmhead"] = {
+            "value": t["tokens"] / (t["ms"] * 1e-3), "unit": "token-logprobs/s", **timing_fields(t),
+            "dtype": "bf16 x bf16 -> f32",
+            "config": {"workload": "config 3: fused lm_head + log-softmax, hidden [4096,1024] x W [151936,1024] bf16",
+                       "tokens": t["tokens"], "hidden": t["H"], "vocab": V, "temperature": 1.0},
+            "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("fused_lmhead_config3"), "fused_lmhead_dma_kernel")}
+        done("fused_lmhead")
+    if "config4" in only:
+        t = bench_fused(dev, K, W, n=16 * 1024, H=2560, temperature=0.7, lengths=(16, 1024, 128, 1024), seed=444)
+        legs["config4_fused_varlen"] = {
+            "value": t["valid"] / (t["ms"] * 1e-3), "unit": "token-logprobs/s", **timing_fields(t),
+            "dtype": "bf16 x bf16 -> f32",
+            "config": {"workload": "config 4: fused lm_head + log-softmax, hidden [16x1024, 2560] x W [151936, 2560] bf16, "
+                                   "temperature 0.7, sequence lengths~U[128,1024] as a padding mask (FLOP counted on valid tokens)",
+                       "tokens": t["tokens"], "valid_tokens": t["valid"], "hidden": t["H"], "vocab": V, "temperature": 0.7},
+            "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("fused_lmhead_config4"), "fused_lmhead_dma_kernel")}
+        done("config4_fused_varlen")
+    if "config5" in only:
+        t = bench_dual(dev, max(3, K // 4), max(1, W // 4))     # 0.1 s per step: a quarter of the steps
+        legs["config5_grpo_dual"] = {
+            "value": t["tokens"] / (t["ms"] * 1e-3), "unit": "tokens/s (lp, ref_lp, k3, entropy each)", **timing_fields(t),
+            "steps": max(3, K // 4), "warmup": max(1, W // 4), "dtype": "bf16 x bf16 -> f32",
+            "config": {"workload": "config 5: GRPO policy + reference dual pass, hidden [32x2048, 4096] x two W [151936, 4096] bf16 "
+                                   "(ref = policy + N(0, 0.002^2)); outputs lp, ref_lp, k3, entropy",
+                       "tokens": t["tokens"], "hidden": t["H"], "vocab": V, "temperature": 1.0},
+            "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("grpo_dual_config5"),
+                                      "fused_lmhead_dma_kernel (two sweeps) + fused_combine_kernel")}
+        done("config5_grpo_dual")
+    if "small" in only:
+        t = bench_fused(dev, K, W, n=64)
+        legs["fused_lmhead_decode_batch"] = {
+            "value": t["tokens"] / (t["ms"] * 1e-3), "unit": "token-logprobs/s", **timing_fields(t),
+            "dtype": "bf16 x bf16 -> f32",
+            "config": {"workload": "fused lm_head + log-softmax at a decode-step batch: hidden [64,1024] x W [151936,1024] bf16",
+                       "tokens": t["tokens"], "hidden": t["H"], "vocab": V},
+            "roofline": hbm_roofline(t["bytes"], t["ms"], traffic_of("fused_lmhead_small_64tokens"), "fused_lmhead_small_kernel")}
+        done("fused_lmhead_decode_batch")
+    if "midsize" in only:   # batches of up to one token tile: W streams once, HBM-bound
+        mid = {}
+        for n, H in ((160, 1024), (256, 1024), (64, 4096), (128, 4096)):
+            t = bench_fused(dev, K, W, n=n, H=H, seed=1000 + n + H)
+            mid[f"{n}x{H}"] = {"ms_per_step": t["ms"], "median_ms": t["median_ms"],
+                               "roofline": hbm_roofline(t["bytes"], t["ms"], None, "fused lm_head sweep + combine")}
+            log(f"midsize {n}x{H}: {t['ms'] * 1e3:.1f} us, {mid[f'{n}x{H}']['roofline']['frac']:.3f} of HBM peak")
+            torch.cuda.empty_cache()
+        worst = min(mid.values(), key=lambda d: d["roofline"]["frac"])
+        legs["fused_lmhead_small_batches"] = {
+            "value": worst["roofline"]["achieved"], "unit": "GB/s (lowest of the shapes)", "ms_per_step": worst["ms_per_step"],
+            "median_ms": worst["median_ms"], "min_ms": worst["median_ms"], "settle_launches": None,
+            "dtype": "bf16 x bf16 -> f32",
+            "config": {"workload": "fused lm_head + log-softmax where W streams once: tokens x hidden in {160x1024, 256x1024, "
+                                   "64x4096, 128x4096}, V = 151936", "shapes": mid},
+            "roofline": worst["roofline"]}
+    if "decode" in only:
+        t = bench_decode(dev, K, W)
+        legs["decode_sampler"] = {
+            "value": t["rows"] / (t["ms"] * 1e-3), "unit": "sampled tokens/s", **timing_fields(t), "dtype": "f32",
+            "config": {"workload": "one decode step: top-k sampling + log-prob + argmax, "
+                                   "fp32 logits [64, 151936] (config 1's shape), top_k 20",
+                       "rows": t["rows"], "top_k": t["top_k"], "vocab": V},
+            "roofline": hbm_roofline(t["bytes"], t["ms"], traffic_of("row_sample_decode_64rows"),
+                                     "row_sample_kernel<f32> + row_sample_combine_kernel")}
+        done("decode_sampler")
+    if "lora" in only:
+        t = bench_lora(dev, K, W)
+        legs["lora_merge"] = {
+            "value": t["jobs"] / (t["ms"] * 1e-3), "unit": "weight matrices merged/s", **timing_fields(t), "dtype": "bf16",
+            "config": {"workload": "UpdateWeights at Qwen3-0.6B's shape: 28 layers x (qkv, gate_up, down), LoRA rank 8",
+                       "matrices": t["jobs"], "rank": t["rank"]},
+            "roofline": hbm_roofline(t["bytes"], t["ms"], traffic_of("lora_merge_qwen3_0.6b"), "lora_merge_kernel<1>")}
+        done("lora_merge")
     cpu = None if args.no_cpu else cpu_baseline()
 
     line = {
         "metric": "token-logprobs/sec + % HBM/MFMA peak at V=151936, Qwen3-0.6B shape",
-        "unit": "token-logprobs/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "data": "synthetic", "dtype": "f32",
+        "n_gpus": 1, "steps": K, "warmup": W,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "data": "synthetic",
     }
-    if row is not None and args.row_variant == "all":
-        row["ms_mask"], row["gbs_mask"], row["bytes_mask"], row["n_valid"] = (row["ms_all"], row["gbs_all"],
-                                                                              row["bytes_all"], row["rows"])
-    if row is not None:
-        line.update({
-            "value": row["n_valid"] / (row["ms_mask"] * 1e-3),
-            "ms_per_step": row["ms_mask"],
-            "config": {"workload": "config 2: row log-softmax + target gather, bf16 logits [8x512, 151936], "
-                                   "padding mask lengths~U[64,512], fp32 out",
-                       "rows": row["rows"], "valid_rows": row["n_valid"], "vocab": V, "temperature": 1.0},
-            "roofline": {"bound": "hbm", "achieved": row["gbs_mask"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": row["gbs_mask"] / HBM_PEAK_GBS,
-                         "traffic": TRAFFIC_ROW_ALL if args.row_variant == "all" else TRAFFIC_ROW_MASKED,
-                         "kernel": "row_logprob_kernel<bf16>", "bytes_per_launch": row["bytes_mask"]},
-        })
-        if args.row_variant == "all":
-            line["config"]["workload"] = line["config"]["workload"].replace(
-                "padding mask lengths~U[64,512]", "padding mask NOT applied (all 4096 rows read)")
-        if args.row_variant == "both":
-            line["all_rows"] = {"value": row["rows"] / (row["ms_all"] * 1e-3), "ms_per_step": row["ms_all"],
-                                "config": {"workload": "config 2 without the padding mask: all 4096 rows read"},
-                                "roofline": {"bound": "hbm", "achieved": row["gbs_all"], "peak": HBM_PEAK_GBS,
-                                             "unit": "GB/s", "frac": row["gbs_all"] / HBM_PEAK_GBS, "traffic": TRAFFIC_ROW_ALL,
-                                             "bytes_per_launch": row["bytes_all"]}}
-    if fused is not None:
-        f = {"value": fused["tokens"] / (fused["ms"] * 1e-3), "unit": "token-logprobs/s", "ms_per_step": fused["ms"],
-             "dtype": "bf16 x bf16 -> f32",
-             "config": {"workload": "config 3: fused lm_head + log-softmax, hidden [4096,1024] x W [151936,1024] bf16",
-                        "tokens": fused["tokens"], "hidden": fused["H"], "vocab": V},
-             "roofline": {"bound": "mfma", "achieved": fused["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
-                          "unit": "TFLOP/s", "frac": fused["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": TRAFFIC_FUSED_CFG3,
-                          "kernel": "fused_lmhead_dma_kernel", "flop_per_launch": fused["flop"]}}
-        if row is None:
-            line.update({"value": f["value"], "ms_per_step": f["ms_per_step"], "config": f["config"],
-                         "roofline": f["roofline"], "dtype": "f32"})
-        else:
-            line["fused_lmhead"] = f
-    if small is not None:
-        nbytes = V * small["H"] * 2 + small["tokens"] * small["H"] * 2
-        gbs = nbytes / (small["ms"] * 1e-3) / 1e9
-        d = {"value": small["tokens"] / (small["ms"] * 1e-3), "unit": "token-logprobs/s", "ms_per_step": small["ms"],
-             "dtype": "bf16 x bf16 -> f32",
-             "config": {"workload": "fused lm_head + log-softmax at a decode-step batch: hidden [64,1024] x W [151936,1024] bf16",
-                        "tokens": small["tokens"], "hidden": small["H"], "vocab": V},
-             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                          "traffic": TRAFFIC_FUSED_SMALL_64, "kernel": "fused_lmhead_small_kernel", "bytes_per_launch": nbytes}}
-        if row is None and fused is None:
-            line.update({"value": d["value"], "unit": d["unit"], "ms_per_step": d["ms_per_step"], "config": d["config"],
-                         "roofline": d["roofline"]})
-        else:
-            line["fused_lmhead_decode_batch"] = d
-    if decode is not None:
-        gbs = decode["bytes"] / (decode["ms"] * 1e-3) / 1e9
-        d = {"value": decode["rows"] / (decode["ms"] * 1e-3), "unit": "sampled tokens/s",
-             "ms_per_step": decode["ms"], "dtype": "f32",
-             "config": {"workload": "one decode step: top-k sampling + log-prob + argmax, "
-                                    "fp32 logits [64, 151936] (config 1's shape), top_k 20",
-                        "rows": decode["rows"], "top_k": decode["top_k"], "vocab": V},
-             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": gbs / HBM_PEAK_GBS, "traffic": TRAFFIC_DECODE_64,
-                          "kernel": "row_sample_kernel<f32> + row_sample_combine_kernel",
-                          "bytes_per_launch": decode["bytes"]}}
-        if row is None and fused is None:
-            line.update({"value": d["value"], "unit": d["unit"], "ms_per_step": d["ms_per_step"], "config": d["config"],
-                         "roofline": d["roofline"]})
-        else:
-            line["decode_sampler"] = d
-    if lora is not None:
-        gbs = lora["bytes"] / (lora["ms"] * 1e-3) / 1e9
-        d = {"value": lora["jobs"] / (lora["ms"] * 1e-3), "unit": "weight matrices merged/s", "ms_per_step": lora["ms"],
-             "dtype": "bf16",
-             "config": {"workload": "UpdateWeights at Qwen3-0.6B's shape: 28 layers x (qkv, gate_up, down), LoRA rank 8",
-                        "matrices": lora["jobs"], "rank": lora["rank"]},
-             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                          "traffic": TRAFFIC_LORA_06B, "kernel": "lora_merge_kernel<1>", "bytes_per_launch": lora["bytes"]}}
-        if row is None and fused is None and decode is None:
-            line.update({"value": d["value"], "unit": d["unit"], "ms_per_step": d["ms_per_step"], "config": d["config"],
-                         "roofline": d["roofline"], "dtype": "bf16"})
-        else:
-            line["lora_merge"] = d
+    first = next(iter(legs))
+    line.update(legs[first])                 # headline = config 2 with its mask, unless --only left it out
+    line["unit"] = legs[first]["unit"]
+    for name, obj in legs.items():
+        if name != first:
+            line[name] = obj
     if cpu is not None:
         line["cpu_baseline"] = cpu
     print(json.dumps(line), flush=True)

@@ -2,7 +2,7 @@
  *
  * Every entry point is a plain-C function over device pointers and sizes.  The
  * caller owns every buffer (inputs, outputs, workspace); the library never
- * allocates, frees or keeps a pointer.  Launches are asynchronous on the HIP
+ * allocates, frees or keeps a caller's pointer.  Launches are asynchronous on the HIP
  * stream passed as `stream` (a hipStream_t cast to void*; NULL = default
  * stream) - the caller synchronises, which mirrors MLX's lazy evaluation forced
  * by mx.eval (mlx-impl/node.py:456).  Return value: 0 on success, a negative
@@ -16,6 +16,13 @@
  *                    reference's slicing by completion length (node.py:449).
  *   temperature      > 0 and finite; the reference maps 0 to 1.0 before the call
  *                    (`temperature or 1.0`, node.py:451) and so must the caller.
+ *   argmax           first maximum of the row (lowest id among equal values).  The row and sampler
+ *                    kernels compare the logits themselves.  The fused kernels compare the fp32 logits
+ *                    they accumulate (bf16 x bf16 products summed in fp32, in the MFMA's order): the
+ *                    id returned is the first maximum of THOSE numbers, so it equals the argmax of the
+ *                    exact logits whenever the top two differ by more than the fp32 summation error
+ *                    (about H * 2^-24 * max|h| * max|w|) and otherwise names a logit within that
+ *                    error of the maximum.  NaN logits are never the maximum.
  *   out_*            float32 per row; any of out_lse / out_entropy / out_argmax may
  *                    be NULL.  lse and entropy are in nats of the temperature-scaled
  *                    logits z = x / temperature.
@@ -128,8 +135,18 @@ int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows
  *           the final RMSNorm of model.py:536 is the caller's)
  *   weight  bf16 [V, H] row-major (the tied embedding matrix), row stride weight_stride
  * Products are exact bf16 x bf16, accumulated in fp32; logits are NOT rounded to bf16.
- * Needs H % 8 == 0 and 16-byte aligned rows.
+ * Needs H % 8 == 0 and 16-byte aligned rows; row strides below 2^31 elements.  With H % 64 != 0
+ * (the generic kernel, 32-bit byte offsets) hidden and weight must each span less than 4 GiB.
+ *
+ * Process-wide state of the library, all of it caches that do not change results: the CU count
+ * of the first GPU used (one workgroup per CU for batches of up to 128 tokens), a flag per large-LDS
+ * kernel ("dynamic LDS limit raised"), the device address of tome_row_logprob_noalloc's array,
+ * and the selector below.
  */
+/* Testing and tuning hook, no counterpart in the reference: kind 0 / 1 makes the fused entry points take
+ * the generic / LDS-DMA sweep kernel wherever its shape rules allow, -1 (the default) picks by shape.
+ * Process-wide; set it while no call of this library is running. */
+void tome_select_fused_kernel(int kind);
 size_t tome_fused_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V);
 int tome_fused_lmhead_logprob(const void* hidden, const void* weight, int64_t n_tokens, int64_t H,
                               int64_t V, int64_t hidden_stride, int64_t weight_stride,
@@ -218,6 +235,16 @@ typedef struct TomeLoraJob {
 size_t tome_lora_merge_workspace(const TomeLoraJob* jobs, int64_t n_jobs);
 int tome_lora_merge(const TomeLoraJob* jobs, int64_t n_jobs, void* workspace, size_t workspace_bytes,
                     void* stream);
+
+/* ---- Measurement probe ---------------------------------------------------------------
+ * No counterpart in the reference.  Runs the LDS -> MFMA inner loop of the fused kernel (256 x 256
+ * workgroup tile, 16x16x32 bf16 MFMA, same fragment reads) on `operands` - 64 KiB of bf16 that each
+ * workgroup copies into LDS once - for `steps` 64-wide K slabs: no global loads in the loop, no
+ * barrier, no epilogue.  One launch does n_workgroups * steps * 2 * 256 * 256 * 64 FLOP; timing it
+ * with random operands gives the bf16 MFMA rate this part sustains under its power limit, which
+ * bench.py reports beside the published peak.  `sink` receives n_workgroups * 512 floats.
+ */
+int tome_probe_mfma_ceiling(const void* operands, int n_workgroups, int steps, float* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -210,14 +210,16 @@ def rms_norm_bf16(x: np.ndarray, weight: np.ndarray, eps: float = 1e-6) -> np.nd
 def top_k_rows(x: np.ndarray, top_k: int = 20):
     """The ``top_k`` largest entries of each row: ``mx.argpartition(scaled_logits, size - top_k)[-top_k:]``
     (mlx-impl/node.py:902; temperature > 0 does not change the set), returned ordered by value
-    descending, equal values by ascending index.  NaN entries are never candidates; a row with fewer
-    than ``top_k`` candidates is padded with index -1.  Returns (idx int32 [rows, top_k], val float64)."""
+    descending, equal values by ascending index.  NaN and -inf entries are never candidates (a -inf
+    logit has probability zero under the categorical of node.py:906, so leaving it out changes no draw);
+    a row with fewer than ``top_k`` candidates is padded with index -1.
+    Returns (idx int32 [rows, top_k], val float64)."""
     x64 = to_f64(x)
     rows, V = x64.shape
     idx = np.full((rows, top_k), -1, dtype=np.int32)
     val = np.zeros((rows, top_k), dtype=np.float64)
     for r in range(rows):
-        cand = np.flatnonzero(~np.isnan(x64[r]))
+        cand = np.flatnonzero(x64[r] > -np.inf)                      # drops NaN too
         order = cand[np.lexsort((cand, -x64[r, cand]))][:top_k]     # value descending, then index ascending
         idx[r, :len(order)] = order
         val[r, :len(order)] = x64[r, order]
@@ -231,14 +233,15 @@ def sample_top_k(x: np.ndarray, uniforms, temperature: float, top_k: int = 20):
     over ``top_logits = (logits / temperature)[top_indices]`` (node.py:899-907) taken as the inverse
     CDF of softmax(top_logits) at ``uniforms[r]`` in [0, 1), candidates in the order of
     ``top_k_rows``.  Returns (token int32 [rows], lp float64 [rows]) where lp is the log-prob of the
-    token under the full softmax at ``temperature or 1.0`` (node.py:590,605)."""
+    token under the full softmax at ``temperature or 1.0`` (node.py:590,605).  A row without any
+    candidate (all -inf / NaN) yields token -1 and lp NaN."""
     x64 = to_f64(x)
     rows = x64.shape[0]
     idx, val = top_k_rows(x, top_k)
     tok = np.empty(rows, dtype=np.int32)
     for r in range(rows):
         n = int((idx[r] >= 0).sum())
-        if temperature == 0 or uniforms is None:
+        if n == 0 or temperature == 0 or uniforms is None:
             tok[r] = idx[r, 0]
             continue
         z = val[r, :n] / float(temperature)
@@ -246,7 +249,9 @@ def sample_top_k(x: np.ndarray, uniforms, temperature: float, top_k: int = 20):
         cdf = np.cumsum(p)
         j = int(np.searchsorted(cdf, float(uniforms[r]) * cdf[-1], side="right"))
         tok[r] = idx[r, min(j, n - 1)]
-    lp = logprob_rows(x64, tok, float(temperature) or 1.0)
+    with np.errstate(invalid="ignore"):
+        lp = logprob_rows(x64, np.maximum(tok, 0), float(temperature) or 1.0)
+    lp = np.where(tok < 0, np.nan, lp)
     return tok, lp
 
 

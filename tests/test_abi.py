@@ -86,7 +86,9 @@ def test_argument_checks_run_on_host():
     assert fused(H=0) == -3 and fused(hs=32) == -3 and fused(T=0.0) == -5
     assert fused(H=60, hs=60, ws=60) == -6 and fused(h=P + 2) == -6
     assert fused(h=None) == -1 and fused(n=0) == 0
-    assert fused(n=1 << 20, H=4096, hs=4096, ws=4096) == -3          # > 4 GiB of hidden
+    assert fused(n=1 << 25, H=72, hs=72, ws=72) == -3                # generic kernel (H % 64 != 0): > 4 GiB of hidden
+    assert fused(n=1 << 20, H=4096, hs=4096, ws=4096) == -4          # the other kernels take it (64-bit addresses)
+    assert fused(hs=1 << 31) == -3 and fused(ws=1 << 40) == -3       # strides are 32-bit byte counts
     assert fused() == -4                                             # workspace missing
     norm = lambda **k: lib.tome_norm_lmhead_logprob(P, k.get("nw", P), k.get("eps", 1e-6), P, 8, k.get("H", 64), 100, 64, 64,
                                                     P, None, 1.0, P, None, None, None, None, 0, None)

@@ -112,20 +112,27 @@ def test_sampler_law_of_the_draw(dev):
     assert set(got.tolist()) <= set(idx[0].tolist())
 
 
-def test_sampler_masks_nan_and_short_rows(dev):
-    V = 4100
-    x = np.random.default_rng(2).standard_normal((4, V)).astype(np.float32)
+@pytest.mark.parametrize("V", [4100, 151936])
+def test_sampler_masks_nan_and_short_rows(dev, V):
+    x = np.random.default_rng(2).standard_normal((5, V)).astype(np.float32)
     x[1, 10] = np.nan                                # NaN is never a candidate, but poisons the row's lse
     x[2, :] = -np.inf
-    x[2, [5, 9]] = [1.0, 2.0]                        # only two finite logits
-    valid = torch.tensor([1, 1, 1, 0], dtype=torch.int32, device=dev)
-    got = tome_amd.sample_tokens(torch.from_numpy(x).to(dev), 1.0, 4, uniforms=[0.5, 0.5, 0.9, 0.5], row_valid=valid, want_topk=True)
-    tki = got.topk_idx.cpu().numpy()
+    x[2, [5, 9]] = [1.0, 2.0]                        # only two logits above -inf: fewer than top_k
+    x[4, :] = -np.inf                                # no candidate at all
+    valid = torch.tensor([1, 1, 1, 0, 1], dtype=torch.int32, device=dev)
+    got = tome_amd.sample_tokens(torch.from_numpy(x).to(dev), 1.0, 4, uniforms=[0.5, 0.5, 0.9, 0.5, 0.5], row_valid=valid,
+                                 want_topk=True)
+    tki, tkl = got.topk_idx.cpu().numpy(), got.topk_logit.cpu().numpy()
+    tok, lp = got.token.cpu().numpy(), got.lp.cpu().numpy()
     want_idx, _ = oracle.top_k_rows(x.astype(np.float64), 4)
-    np.testing.assert_array_equal(tki[0], want_idx[0])
-    assert 10 not in tki[1] and np.isnan(got.lp.cpu().numpy()[1])
-    assert tki[2, :2].tolist() == [9, 5] and got.token.cpu().numpy()[2] == 5          # masses e^2 : e^1 -> 0.9 falls on id 5
-    assert got.token.cpu().numpy()[3] == -1 and got.lp.cpu().numpy()[3] == 0 and (tki[3] == -1).all()
+    np.testing.assert_array_equal(tki[[0, 2, 4]], want_idx[[0, 2, 4]])                # -inf logits are not listed
+    assert 10 not in tki[1] and np.isnan(lp[1])
+    assert tki[2].tolist() == [9, 5, -1, -1] and tkl[2].tolist() == [2.0, 1.0, 0.0, 0.0]
+    assert tok[2] == 5                                                                 # masses e^2 : e^1 -> 0.9 falls on id 5
+    want_tok, want_lp = oracle.sample_top_k(x[2:3].astype(np.float64), [0.9], 1.0, 4)
+    assert tok[2] == want_tok[0] and abs(lp[2] - want_lp[0]) < 1e-4
+    assert tok[3] == -1 and lp[3] == 0 and (tki[3] == -1).all()
+    assert tok[4] == -1 and np.isnan(lp[4]) and (tki[4] == -1).all()                  # all -inf: no token
 
 
 def test_sampler_strided_and_unaligned_rows(dev):

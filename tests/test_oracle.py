@@ -268,10 +268,18 @@ def test_top_k_rows_against_argpartition_and_bruteforce():
     t = np.zeros((1, 12)); t[0, [7, 2, 9]] = 5.0; t[0, [4, 1, 11, 6]] = 3.0
     idx, _ = oracle.top_k_rows(t, 5)
     assert idx[0].tolist() == [2, 7, 9, 1, 4]
-    # NaN is never a candidate; short rows are padded with -1
-    s = np.array([[np.nan, 1.0, -np.inf, 2.0]])
+    # NaN and -inf are never candidates (a -inf logit has probability zero in the draw of node.py:906, so the
+    # law of the draw is the same with or without it); short rows are padded with -1
+    s = np.array([[np.nan, 1.0, -np.inf, 2.0], [-np.inf] * 4])
     idx, val = oracle.top_k_rows(s, 4)
-    assert idx[0].tolist() == [3, 1, 2, -1] and val[0, 0] == 2.0
+    assert idx[0].tolist() == [3, 1, -1, -1] and val[0, 0] == 2.0 and idx[1].tolist() == [-1] * 4
+    # fewer finite logits than top_k: the draw is over the finite ones with their softmax masses (e^2 : e^1)
+    short = np.full((1, 50), -np.inf); short[0, [5, 9]] = [1.0, 2.0]
+    p9 = math.exp(2.0) / (math.exp(2.0) + math.exp(1.0))
+    assert [int(oracle.sample_top_k(short, [u], 1.0, 20)[0][0]) for u in (0.0, p9 - 1e-9, p9 + 1e-9, 0.999)] == [9, 9, 5, 5]
+    # no candidate at all: token -1, lp NaN
+    tok, lp = oracle.sample_top_k(s[1:], [0.5], 1.0, 4)
+    assert tok[0] == -1 and np.isnan(lp[0])
 
 
 def test_sample_top_k_law_and_limits():

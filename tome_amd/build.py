@@ -8,7 +8,7 @@ import sys
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libtome_logprob.so")
-SOURCES = ["capi.hip", "row_logprob.hip", "row_sample.hip", "full_log_softmax.hip", "fused_lmhead.hip", "lora_merge.hip"]
+SOURCES = ["capi.hip", "row_logprob.hip", "row_sample.hip", "full_log_softmax.hip", "fused_lmhead.hip", "lora_merge.hip", "mfma_probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc",

@@ -25,6 +25,8 @@ hipError_t row_sample_launch(const void* logits, int dtype, int64_t rows, int64_
                              int32_t* out_topk_idx, float* out_topk_logit, void* workspace, hipStream_t stream);
 size_t row_sample_workspace_bytes(int64_t rows, int64_t V, int dtype_vec, int top_k);
 size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights, bool with_norm);
+bool fused_needs_32bit_extents(int64_t n_tokens, int64_t H, int64_t V);
+void fused_force_kernel(int kind);
 hipError_t fused_lmhead_launch(const void* hidden, const void* norm_weight, float norm_eps, const void* w0,
                                const void* w1, int64_t n_tokens, int64_t H, int64_t V, int64_t hidden_stride,
                                int64_t weight_stride, const int32_t* targets,
@@ -36,6 +38,7 @@ hipError_t fused_pair_launch(const void* hidden, const void* hidden_ref, const v
                              int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
                              const int32_t* row_valid, float temperature, float* out_lp, float* out_entropy,
                              float* out_ref_lp, float* out_k3, void* workspace, hipStream_t stream);
+hipError_t mfma_probe_launch(const void* operands, int n_workgroups, int steps, float* sink, hipStream_t stream);
 struct LoraJobHost;
 hipError_t lora_merge_launch(const LoraJobHost* jobs, int n_jobs, void* workspace, hipStream_t stream);
 size_t lora_workspace_bytes(const LoraJobHost* jobs, int n_jobs);
@@ -175,8 +178,12 @@ static int check_fused(const void* hidden, const void* w, int64_t n_tokens, int6
                        int64_t hidden_stride, int64_t weight_stride, const int32_t* targets, float temperature) {
   if (n_tokens < 0 || H <= 0 || V <= 0 || hidden_stride < H || weight_stride < H) return TOME_E_SHAPE;
   if (V > (int64_t)0x7fffffff || n_tokens > (int64_t)0x7fffffff || H > (int64_t)1 << 20) return TOME_E_SHAPE;
-  // The kernel addresses both matrices with 32-bit byte offsets.
-  if (n_tokens * hidden_stride * 2 >= ((int64_t)1 << 32) || V * weight_stride * 2 >= ((int64_t)1 << 32))
+  // Row strides travel as 32-bit byte counts (checked before anything is multiplied by them).
+  if (hidden_stride > (int64_t)0x7fffffff || weight_stride > (int64_t)0x7fffffff) return TOME_E_SHAPE;
+  // The generic kernel (H % 64 != 0) also addresses both matrices with 32-bit byte offsets: each must stay
+  // below 4 GiB there.  The other kernels use 64-bit addresses.
+  if (tome::fused_needs_32bit_extents(n_tokens, H, V) &&
+      (n_tokens * hidden_stride * 2 >= ((int64_t)1 << 32) || V * weight_stride * 2 >= ((int64_t)1 << 32)))
     return TOME_E_SHAPE;
   if (bad_temperature(temperature)) return TOME_E_TEMPERATURE;
   if (n_tokens == 0) return TOME_OK;
@@ -186,6 +193,8 @@ static int check_fused(const void* hidden, const void* w, int64_t n_tokens, int6
     return TOME_E_ALIGN;
   return TOME_OK;
 }
+
+void tome_select_fused_kernel(int kind) { tome::fused_force_kernel(kind < 0 || kind > 1 ? -1 : kind); }
 
 size_t tome_fused_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V) {
   if (n_tokens <= 0 || H <= 0 || V <= 0) return 0;
@@ -277,6 +286,13 @@ int tome_grpo_pair(const void* hidden_policy, const void* hidden_ref, const void
                                             H, V, hidden_stride, weight_stride, targets, row_valid, temperature,
                                             out_lp, out_entropy, out_ref_lp, out_k3, workspace,
                                             static_cast<hipStream_t>(stream)));
+}
+
+int tome_probe_mfma_ceiling(const void* operands, int n_workgroups, int steps, float* sink, void* stream) {
+  if (!operands || !sink) return TOME_E_NULL;
+  if (n_workgroups <= 0 || n_workgroups > 65536 || steps <= 0 || steps > (1 << 24)) return TOME_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(operands) % 16 != 0) return TOME_E_ALIGN;
+  return hip_result(tome::mfma_probe_launch(operands, n_workgroups, steps, sink, static_cast<hipStream_t>(stream)));
 }
 
 static int check_lora_jobs(const TomeLoraJob* jobs, int64_t n_jobs) {

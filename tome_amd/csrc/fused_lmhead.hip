@@ -27,7 +27,7 @@
 //   * Masked tokens are compacted first (compact_rows_kernel); token tiles are built from
 //     the compacted index list, so masked rows cost no FLOPs and no HBM traffic.
 #include "common.hpp"
-#include <cstdlib>
+#include <atomic>
 #include <type_traits>
 
 namespace tome {
@@ -181,7 +181,7 @@ __device__ __forceinline__ u32x4 ld16(__amdgpu_buffer_rsrc_t r, uint32_t lane_of
 // running states.  Accumulator element e of block i holds vocab row
 //   vw0 + i*32 + 8*(e/4) + 4*lh + e%4        (vw0 = first vocab row of this wave's tile)
 // for the token this lane owns in block column j.
-template <bool ENT, int NBV, int NBT>
+template <bool ENT, bool AMAX, int NBV, int NBT>
 __device__ __forceinline__ void fold_tile(f32x16 (&acc)[NBV][NBT], RowStat (&st)[NBT], float (&tx)[NBT],
                                           const int (&tgt)[NBT], int vw0, int lh, bool partial_tile, int V,
                                           float scale) {
@@ -195,6 +195,7 @@ __device__ __forceinline__ void fold_tile(f32x16 (&acc)[NBV][NBT], RowStat (&st)
         for (int j = 0; j < NBT; ++j) acc[i][j][e] = dead ? -INFINITY : acc[i][j][e];
       }
   }
+  const int vlane = vw0 + 4 * lh;  // first vocab row this lane holds in block 0
 #pragma unroll
   for (int j = 0; j < NBT; ++j) {
     // One scheduling region per token block: otherwise all accumulator reads of all blocks are
@@ -210,21 +211,25 @@ __device__ __forceinline__ void fold_tile(f32x16 (&acc)[NBV][NBT], RowStat (&st)
 #pragma unroll
         for (int e = 0; e < 16; ++e) tx[j] = (want == i * 16 + e) ? acc[i][j][e] : tx[j];
     }
-    float bm[NBV];  // per 32-row block maximum
-#pragma unroll
-    for (int i = 0; i < NBV; ++i) {
-      float m = acc[i][j][0];
-#pragma unroll
-      for (int e = 1; e < 16; e += 2) m = raw_max3(m, acc[i][j][e], e + 1 < 16 ? acc[i][j][e + 1] : acc[i][j][e]);
-      bm[i] = m;
-    }
     float cm = st[j].mx;
     int bi = st[j].bi;
 #pragma unroll
     for (int i = 0; i < NBV; ++i) {
-      const bool up = bm[i] > cm;
-      bi = up ? (vw0 + i * 32) : bi;  // first row of the 32-row block
-      cm = raw_max(cm, bm[i]);
+      if constexpr (AMAX) {
+        // The running maximum carries the vocab row of the element that set it.  A lane meets its rows in
+        // ascending order and only a strictly larger value replaces the holder, so the first maximum stays.
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float x = acc[i][j][e];
+          bi = x > cm ? vlane + i * 32 + 8 * (e / 4) + (e % 4) : bi;
+          cm = raw_max(cm, x);
+        }
+      } else {
+        float m = acc[i][j][0];
+#pragma unroll
+        for (int e = 1; e < 16; e += 2) m = raw_max3(m, acc[i][j][e], e + 1 < 16 ? acc[i][j][e + 1] : acc[i][j][e]);
+        cm = raw_max(cm, m);
+      }
     }
     const float resc = fast_exp2((st[j].mx - cm) * scale);
     const float m = cm * scale;
@@ -274,7 +279,7 @@ __device__ __forceinline__ void write_partials(RowStat (&st)[NBT], float (&tx)[N
   }
 }
 
-template <bool ENT>
+template <bool ENT, bool AMAX>
 __global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) {
   __shared__ __attribute__((aligned(16))) char lds[(kBV + kBT) * kPitch];
   char* ldsA = lds;
@@ -380,7 +385,7 @@ __global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) 
       }
     }
 
-    fold_tile<ENT>(acc, st, tx, tgt, v0 + wave_v * kWaveV, lh, v0 + kBV > a.V, a.V, a.scale);
+    fold_tile<ENT, AMAX>(acc, st, tx, tgt, v0 + wave_v * kWaveV, lh, v0 + kBV > a.V, a.V, a.scale);
   }
 
   write_partials(st, tx, a.partials, t0 + wave_t * kWaveT, n_valid, split * kPartsPerSplit + wave_v,
@@ -411,6 +416,7 @@ __device__ __forceinline__ void fold_tile16(f32x4v (&acc)[NBV][NBT], RowStat (&s
         for (int j = 0; j < NBT; ++j) acc[i][j][e] = dead ? -INFINITY : acc[i][j][e];
       }
   }
+  const int vlane = vw0 + 4 * g;  // first vocab row this lane holds in block 0
 #pragma unroll
   for (int j = 0; j < NBT; ++j) {
     __builtin_amdgcn_sched_barrier(0);  // one scheduling region per token block (register pressure)
@@ -428,12 +434,22 @@ __device__ __forceinline__ void fold_tile16(f32x4v (&acc)[NBV][NBT], RowStat (&s
     int bi = st[j].bi;
 #pragma unroll
     for (int i = 0; i < NBV; ++i) {
-      const float bm = raw_max3(acc[i][j][0], acc[i][j][1], raw_max(acc[i][j][2], acc[i][j][3]));
-      if constexpr (AMAX) {  // two more VALU operations per block: only when the argmax is asked for
-        const bool up = bm > cm;
-        bi = up ? (vw0 + i * 16) : bi;  // first row of the 16-row block
+      if constexpr (AMAX) {
+        // Seven more VALU operations per block, only when the argmax is asked for: the block maximum comes
+        // with the position of its first holder, and the running maximum carries the vocab row of the
+        // element that set it.  Only a strictly larger value replaces the holder and a lane meets its rows in
+        // ascending order, so the sweep itself names the first maximum of the fp32 logits it computed.
+        const float x0 = acc[i][j][0], x1 = acc[i][j][1], x2 = acc[i][j][2], x3 = acc[i][j][3];
+        const float m01 = raw_max(x0, x1), m23 = raw_max(x2, x3);
+        const int e01 = x1 > x0 ? 1 : 0, e23 = x3 > x2 ? 3 : 2;
+        const int e = m23 > m01 ? e23 : e01;
+        const float bm = raw_max(m01, m23);
+        bi = bm > cm ? vlane + i * 16 + e : bi;
+        cm = raw_max(cm, bm);
+      } else {
+        const float bm = raw_max3(acc[i][j][0], acc[i][j][1], raw_max(acc[i][j][2], acc[i][j][3]));
+        cm = raw_max(cm, bm);
       }
-      cm = raw_max(cm, bm);
     }
     const float resc = fast_exp2((st[j].mx - cm) * scale);
     const float m = cm * scale;
@@ -522,18 +538,29 @@ __device__ __forceinline__ void write_partials16(RowStat (&st)[NBT], float (&tx)
 constexpr int k2BV = 256, k2WG = 512;
 constexpr int k2BK = 64;
 constexpr int k2RowBytes = k2BK * 2;                     // 128: one cache line
-constexpr int dma_slabs(int nbt) { return nbt == 4 ? 2 : 3; }  // slab buffers: as many as fit the 160 KB of LDS
+// Slab buffers, as many as fit the 160 KB of LDS: two for the 256-token tile (64 KB per slab), three otherwise.
+// The W halves and the hidden halves form two rings of that depth.
+constexpr int dma_bufs(int nbt) { return nbt == 4 ? 2 : 3; }
+// With two buffers a slab's request is issued in three portions - in the last quarter of the step that frees
+// its buffer, and in the first two quarters of the next step - instead of all at once: right after a barrier
+// all eight waves are at the same point, and 64 requests issued together queue up in the memory pipeline
+// while the waves that issued them cannot issue their MFMAs.
+constexpr int kIssueQ4 = 4, kIssueQ1 = 2;   // instructions of the eight in the last / first quarter; the rest in the second
 constexpr int k2Loads = k2BV * (k2RowBytes / 16) / k2WG; // DMA instructions per lane and slab for W (4)
 constexpr int k2NBV = kWaveV / 16;                       // 16x16 vocab blocks per wave tile: 8
 static_assert(k2Loads == 4 && k2NBV == 8, "the MFMA/DMA interleave is written for this shape");
 constexpr int dma_tile_tokens(int nbt) { return nbt * 64; }                                   // 4 token waves x nbt x 16
-constexpr int dma_slab_bytes(int nbt) { return (k2BV + dma_tile_tokens(nbt)) * k2RowBytes; }  // 65536 at nbt = 4
-constexpr int dma_lds_bytes(int nbt) { return dma_slabs(nbt) * dma_slab_bytes(nbt); }         // 131072 at nbt = 4
+constexpr int dma_w_bytes() { return k2BV * k2RowBytes; }                                      // 32768
+constexpr int dma_h_bytes(int nbt) { return dma_tile_tokens(nbt) * k2RowBytes; }               // 32768 at nbt = 4
+constexpr int dma_lds_bytes(int nbt) { return dma_bufs(nbt) * (dma_w_bytes() + dma_h_bytes(nbt)); }  // 131072 at nbt = 4
 
+// AUX: cache policy bits of the request (0 = default, 2 = non-temporal).
+template <int AUX = 0>
 __device__ __forceinline__ void dma16(const char* gptr, char* lds_wave_base) {
   __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(gptr),
-                                   (__attribute__((address_space(3))) uint32_t*)lds_wave_base, 16, 0, 0);
+                                   (__attribute__((address_space(3))) uint32_t*)lds_wave_base, 16, 0, AUX);
 }
+constexpr int kDmaAuxW = 0, kDmaAuxH = 0;
 
 // Scheduling pattern: N_READS times (N_MFMA MFMAs, then one LDS read).
 template <int N_MFMA, int N_READS>
@@ -551,10 +578,22 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   constexpr int k2NBT = NBT;                        // 16-token blocks per wave
   constexpr int k2BT = dma_tile_tokens(NBT);        // tokens per workgroup
   constexpr int kWaveTok = NBT * 16;                // tokens per wave
-  constexpr int k2SlabBytes = dma_slab_bytes(NBT);
-  constexpr int k2Slabs = dma_slabs(NBT);           // with three, the barrier of a step no longer waits for the newest request
+  constexpr int kBufs = dma_bufs(NBT);
+  constexpr int kWBytes = dma_w_bytes(), kHBytes = dma_h_bytes(NBT);
+  constexpr int kHBase = kBufs * kWBytes;           // the hidden ring starts behind the W ring
   constexpr int kBLoads = NBT;                      // DMA instructions per lane and slab for the hidden rows
   constexpr int k2DmaPerSlab = k2Loads + kBLoads;   // 8 at NBT = 4
+  // Portions of a request (see kIssueQ4): with three buffers everything goes out in the last quarter.
+  constexpr int kP4 = NBT == 4 ? kIssueQ4 : k2DmaPerSlab;
+  constexpr int kP1 = NBT == 4 ? kIssueQ1 : 0;
+  constexpr int kP2 = k2DmaPerSlab - kP4 - kP1;
+  static_assert(kP4 >= 1 && kP1 >= 0 && kP2 >= 0 && kP1 <= 8 && kP2 <= 8, "portions of the eight instructions");
+  static_assert(kBufs == 2 || kP4 == k2DmaPerSlab, "split requests are written for two buffers");
+  // Requests complete in the order they were issued, so "slab s has landed" is a count of newer instructions that
+  // may still be in flight.  Before a step's barrier (slab step + 1 must be there) those are the whole requests
+  // of the slabs after it; before the loop (slab 0) also the first portion of the newest request.
+  constexpr int kInFlightAtStep = (kBufs - 2) * k2DmaPerSlab;
+  constexpr int kInFlightAtStart = (kBufs - 2) * k2DmaPerSlab + kP4;
 
   const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
   const FusedSchedule sch = a.sched_dev ? *a.sched_dev : a.sched;
@@ -610,21 +649,21 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   // ---- fragment read offsets inside a slab (swizzled): lane group g reads chunk 4*ks + g ----------
   const int swz = (g ^ ((l16 >> 1) & 7)) * 16;  // sub-step k0; k1 is this ^ 64
   const int rdA = (wave_v * kWaveV + l16) * k2RowBytes + swz;
-  const int rdB = k2BV * k2RowBytes + (wave_t * kWaveTok + l16) * k2RowBytes + swz;
+  const int rdB = (wave_t * kWaveTok + l16) * k2RowBytes + swz;
 
   const int nk = a.H / k2BK;
   const int n_steps = (vt1 - vt0) * nk;
   const int64_t slab_rewind = (int64_t)(nk - 1) * k2RowBytes;
-  int i_kt = 0, i_vt = vt0;  // slab the next `issue` will request
-  int issued = 0;            // slabs requested so far; request q lands in buffer q % k2Slabs
+  int i_kt = 0, i_vt = vt0;  // slab the next request fetches
+  int issued = 0;            // slabs requested so far; request q lands in buffers q % kBufs
 
-  // One of the eight DMA instructions of the next request (0-3: W rows; 4-7: hidden rows).
+  // One of the DMA instructions of the next request (0-3: W rows; the others: hidden rows).  Past the last slab
+  // the request is repeated (same addresses, same buffer, identical bytes): it is issued on every step so that
+  // the code has no branch and the wait counts stay static.
   auto issue_piece = [&](int piece) {
-    // Past the last slab the request is repeated (same addresses, same buffer, identical bytes): it is
-    // issued on every step so that the code has no branch and the wait counts stay static.
-    char* dst = smem + ((unsigned)(issued < n_steps ? issued : n_steps - 1) % k2Slabs) * k2SlabBytes + wave * 1024;
-    if (piece < k2Loads) dma16(pa[piece], dst + piece * 8192);
-    else dma16(pb[piece - k2Loads], dst + k2BV * k2RowBytes + (piece - k2Loads) * 8192);
+    const unsigned buf = (unsigned)(issued < n_steps ? issued : n_steps - 1) % kBufs;
+    if (piece < k2Loads) dma16<kDmaAuxW>(pa[piece], smem + buf * kWBytes + wave * 1024 + piece * 8192);
+    else dma16<kDmaAuxH>(pb[piece - k2Loads], smem + kHBase + buf * kHBytes + wave * 1024 + (piece - k2Loads) * 8192);
   };
   auto issue_done = [&]() {
     ++issued;
@@ -642,29 +681,32 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
       if (i_vt < vt1) point_a(i_vt);
     }
   };
-  // Fragments of one K = 32 sub-step of a slab: W blocks [i0, i0 + 4) or the four hidden blocks.
+  // Fragments of one K = 32 sub-step of a slab: W blocks [i0, i0 + 4) or the hidden blocks.
   auto read_a = [&](int slot, int ks, int i0, bf16x8 (&fa)[4]) {
-    const char* slab = smem + ((unsigned)slot % k2Slabs) * k2SlabBytes;
+    const char* slab = smem + ((unsigned)slot % kBufs) * kWBytes;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       fa[i] = *reinterpret_cast<const bf16x8*>(slab + (rdA ^ (ks * 64)) + (i0 + i) * 16 * k2RowBytes);
   };
   auto read_b = [&](int slot, int ks, bf16x8 (&fb)[k2NBT]) {
-    const char* slab = smem + ((unsigned)slot % k2Slabs) * k2SlabBytes;
+    const char* slab = smem + kHBase + ((unsigned)slot % kBufs) * kHBytes;
 #pragma unroll
     for (int j = 0; j < k2NBT; ++j)
       fb[j] = *reinterpret_cast<const bf16x8*>(slab + (rdB ^ (ks * 64)) + j * 16 * k2RowBytes);
   };
 
-  for (int q = 0; q < k2Slabs; ++q) {
+  // Prologue: whole requests for all buffers but the last, and the first portion of the last one's.
+#pragma unroll
+  for (int q = 0; q < kBufs - 1; ++q) {
 #pragma unroll
     for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
     issue_done();
   }
+#pragma unroll
+  for (int piece = 0; piece < kP4; ++piece) issue_piece(piece);
+  if constexpr (kP4 == k2DmaPerSlab) issue_done();
   // Slab 0 has landed (this wave's share): only the requests of the later slabs may still be in flight.
-  if constexpr (NBT == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");        // 1 slab x 8 requests
-  else if constexpr (NBT == 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");  // 2 slabs x 6
-  else asm volatile("s_waitcnt vmcnt(10)" ::: "memory");                          // 2 slabs x 5
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kInFlightAtStart) : "memory");
   __builtin_amdgcn_s_barrier();
 
   bf16x8 fa_lo[4], fa_hi[4], fb0[k2NBT], fb1[k2NBT];
@@ -693,47 +735,64 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
                                                                    0, 0, 0);
   };
   int step = 0;
+  // N times (one MFMA, then one DMA request).
+  auto pair_dma = [](auto n) {
+#pragma unroll
+    for (int q = 0; q < decltype(n)::value; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM (DMA request)
+    }
+  };
   auto do_step = [&](auto fresh) {
     __builtin_amdgcn_sched_barrier(0);
     read_a(step, 0, 4, fa_hi);
+#pragma unroll
+    for (int piece = kP4; piece < kP4 + kP1; ++piece) issue_piece(piece);  // second portion of the request for slab step + 1
     mfma_half(0, fa_lo, fb0, fresh);
-    if constexpr (NBT == 4) pair_reads<2, 4>();
+    if constexpr (NBT == 4) {
+      pair_reads<2, 4>();
+      pair_dma(std::integral_constant<int, kP1>{});
+    }
     __builtin_amdgcn_sched_barrier(0);
     read_a(step, 1, 0, fa_lo);
     read_b(step, 1, fb1);
+#pragma unroll
+    for (int piece = kP4 + kP1; piece < k2DmaPerSlab; ++piece) issue_piece(piece);  // third portion
     mfma_half(4, fa_hi, fb0, fresh);
-    if constexpr (NBT == 4) pair_reads<2, 8>();
+    if constexpr (NBT == 4) {
+      if constexpr (kP2 == 0) {
+        pair_reads<2, 8>();
+      } else {
+        pair_reads<1, 8>();
+        pair_dma(std::integral_constant<int, kP2>{});
+      }
+    }
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (kP4 < k2DmaPerSlab) issue_done();
     read_a(step, 1, 4, fa_hi);
     mfma_half(0, fa_lo, fb1, std::false_type{});
     if constexpr (NBT == 4) pair_reads<2, 4>();
     __builtin_amdgcn_sched_barrier(0);
     // This wave has read all it needs of slab `step` and its share of slab step+1 has landed; after
-    // the (fence-less) barrier both hold for everyone.
-    // (With three buffers the requests of slab step+2 stay in flight across the barrier.)
-    if constexpr (NBT == 4) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    else if constexpr (NBT == 2) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory");
+    // the (fence-less) barrier both hold for everyone.  (With three buffers the request of slab step+2
+    // stays in flight across the barrier.)
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kInFlightAtStep) : "memory");
     __builtin_amdgcn_s_barrier();
     // Last quarter: first fragments of slab step+1 (after the last step a stale buffer, unused) and the
-    // next request, which refills the buffer of slab `step`.  The DMA requests write LDS, so they keep
-    // their program order after the fragment reads.
+    // first portion of the next request, which refills the buffers of slab `step`.  The DMA requests write
+    // LDS, so they keep their program order after the fragment reads.
     __builtin_amdgcn_sched_barrier(0);
     read_a(step + 1, 0, 0, fa_lo);
     read_b(step + 1, 0, fb0);
 #pragma unroll
-    for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
+    for (int piece = 0; piece < kP4; ++piece) issue_piece(piece);
     mfma_half(4, fa_hi, fb1, std::false_type{});
     if constexpr (NBT == 4) {
       pair_reads<1, 8>();
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM (DMA request)
-      }
+      pair_dma(std::integral_constant<int, kP4>{});
     }
     __builtin_amdgcn_sched_barrier(0);
-    issue_done();
+    if constexpr (kP4 == k2DmaPerSlab) issue_done();
     ++step;
   };
 
@@ -895,6 +954,7 @@ struct CompactArgs {
   float* out1;
   float* out2;
   float* out3;
+  float* out4;
   int32_t* out_argmax;
   int n;
   int bt, slots, n_vtiles;  // inputs of the schedule, which this kernel derives from n_valid
@@ -926,6 +986,7 @@ __global__ __launch_bounds__(1024) void compact_rows_kernel(CompactArgs a) {
       if (a.out1) a.out1[r] = 0.f;
       if (a.out2) a.out2[r] = 0.f;
       if (a.out3) a.out3[r] = 0.f;
+      if (a.out4) a.out4[r] = 0.f;
       if (a.out_argmax) a.out_argmax[r] = -1;
     }
   }
@@ -1002,58 +1063,11 @@ struct CombineArgs {
   float* out_ref_lp;
   float* out_k3;
   int32_t* out_argmax;
-  const char* hidden;  // only read when out_argmax is set
-  const int32_t* hidden_index;  // as in FusedArgs
-  const char* weight;
-  uint32_t hidden_stride_b;
-  uint32_t weight_stride_b;
-  int H;
-  int V;
   int n_tokens;
   const FusedSchedule* sched_dev;  // as in FusedArgs
   FusedSchedule sched;
   float scale;
 };
-
-// Greedy token id of one token.  The sweep only records WHICH 32-row vocab block held the
-// row maximum (first block on ties); the 32 logits of that block are recomputed here as
-// fp32 dot products (lanes l and l+32 take the two halves of K) and the first maximum wins.
-__device__ __forceinline__ int argmax_in_block(const CombineArgs& a, int tok, int block0, int lane) {
-  if (block0 < 0 || block0 >= a.V) return 0;  // nothing above the floor was seen
-  const int row = block0 + (lane & 31), half = lane >> 5;
-  float d = -INFINITY;
-  if (row < a.V) {
-    const u32x4* w = reinterpret_cast<const u32x4*>(a.weight + (int64_t)row * a.weight_stride_b);
-    const u32x4* h = reinterpret_cast<const u32x4*>(a.hidden + (int64_t)tok * a.hidden_stride_b);
-    const int n_chunks = a.H / 8, mid = (n_chunks + 1) / 2;
-    float acc = 0.f;
-    for (int c = half ? mid : 0; c < (half ? n_chunks : mid); ++c) {
-      const u32x4 wv = w[c], hv = h[c];
-      acc = fmaf(bf16_lo(wv.x), bf16_lo(hv.x), acc);
-      acc = fmaf(bf16_hi(wv.x), bf16_hi(hv.x), acc);
-      acc = fmaf(bf16_lo(wv.y), bf16_lo(hv.y), acc);
-      acc = fmaf(bf16_hi(wv.y), bf16_hi(hv.y), acc);
-      acc = fmaf(bf16_lo(wv.z), bf16_lo(hv.z), acc);
-      acc = fmaf(bf16_hi(wv.z), bf16_hi(hv.z), acc);
-      acc = fmaf(bf16_lo(wv.w), bf16_lo(hv.w), acc);
-      acc = fmaf(bf16_hi(wv.w), bf16_hi(hv.w), acc);
-    }
-    d = acc;
-  }
-  const float other = __shfl_xor(d, 32, 64);
-  d = row < a.V ? d + other : -INFINITY;  // both halves now hold the full dot product
-  int idx = lane & 31;
-#pragma unroll
-  for (int off = 16; off > 0; off >>= 1) {
-    const float od = __shfl_xor(d, off, 64);
-    const int oi = __shfl_xor(idx, off, 64);
-    if (od > d || (od == d && oi < idx)) {
-      d = od;
-      idx = oi;
-    }
-  }
-  return block0 + idx;
-}
 
 __device__ __forceinline__ void combine_one(const FusedPartial* parts, int n_parts, int lane, float scale,
                                             RowStat& st, float& tx) {
@@ -1092,10 +1106,10 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
     const float mr = sr.mx * a.scale;
     ref_lp = txr == -INFINITY ? __builtin_nanf("") : (fmaf(txr, a.scale, -mr) - fast_log2(sr.s)) * kLn2;
   }
-  int amax = 0;
-  if (a.out_argmax) amax = argmax_in_block(a, a.hidden_index ? a.hidden_index[p] : p, st.bi == 0x7fffffff ? -1 : st.bi, lane);
   if (lane != 0) return;
-  if (a.out_argmax) a.out_argmax[tok] = amax;
+  // The sweep kernels name the element themselves: bi is the vocab row of the first maximum among the fp32
+  // logits they accumulated (0 when nothing above the floor was seen, as a first-maximum scan would say).
+  if (a.out_argmax) a.out_argmax[tok] = st.bi == 0x7fffffff ? 0 : st.bi;
   if (a.out_lp) a.out_lp[tok] = lp;
   if (a.out_lse) a.out_lse[tok] = (m + log2s) * kLn2;
   if (a.out_entropy) a.out_entropy[tok] = (m + log2s - st.w / st.s) * kLn2;
@@ -1111,6 +1125,11 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
 // with the batch.  Decode-sized batches whose hidden states fit the waves' registers take the streaming kernel.
 
 enum FusedKind { kGeneric = 0, kDma = 1, kSmall = 2 };
+
+// Kernel selector for tests and tuning runs: -1 (the default) picks by shape, kGeneric / kDma force that
+// sweep kernel wherever its shape rules allow.  Process-wide; set it while no call is in flight.
+static std::atomic<int> g_forced_kind{-1};
+void fused_force_kernel(int kind) { g_forced_kind.store(kind, std::memory_order_relaxed); }
 
 struct FusedPlan {
   FusedKind kind;
@@ -1173,11 +1192,11 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   p.small_nbt = p.small_ksteps = p.small_waves = 0;
   p.dma_nbt = n_tokens > 128 ? 4 : (n_tokens > 64 ? 2 : 1);
   if (H % k2BK == 0) p.kind = kDma;
-  if (small_shape(n_tokens, H, V, p.small_nbt, p.small_ksteps, p.small_waves)) p.kind = kSmall;
-  if (const char* ov = getenv("TOME_FUSED_KERNEL")) {  // tuning knob: force a path where its shape rules allow
-    if (ov[0] == 'g') p.kind = kGeneric;
-    if (ov[0] == 'd' && H % k2BK == 0) p.kind = kDma;
-  }
+  // The streaming kernel runs one workgroup per CU: without a CU count (no device) the tiled kernels serve.
+  if (small_shape(n_tokens, H, V, p.small_nbt, p.small_ksteps, p.small_waves) && small_wg_count() >= 2) p.kind = kSmall;
+  const int forced = g_forced_kind.load(std::memory_order_relaxed);
+  if (forced == kGeneric) p.kind = kGeneric;
+  if (forced == kDma && H % k2BK == 0) p.kind = kDma;
   p.n_vtiles = 0;
   if (p.kind == kSmall) {
     // One partial per (token, workgroup); one workgroup per CU, at most 512.
@@ -1219,6 +1238,9 @@ static size_t partial_bytes(int64_t n_tokens, int64_t H, int64_t V) {
   return fused_plan(n_tokens, H, V).max_records * sizeof(FusedPartial);
 }
 
+// The generic kernel addresses both matrices through buffer descriptors with 32-bit byte offsets.
+bool fused_needs_32bit_extents(int64_t n_tokens, int64_t H, int64_t V) { return fused_plan(n_tokens, H, V).kind == kGeneric; }
+
 size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weights, bool with_norm) {
   return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, H, V) + normed_bytes(n_tokens, H, with_norm);
 }
@@ -1258,7 +1280,7 @@ static int launch_small(const FusedArgs& a, int waves, hipStream_t stream) {
 }
 
 // Launches the sweep kernel of `plan`.  Returns the number of partials per token it leaves (0 = the
-// schedule's own count), or -1 when the small-batch kernel could not be placed.
+// schedule's own count).
 template <bool ENT>
 static int launch_main(const FusedArgs& a, const FusedPlan& plan, bool want_argmax, hipStream_t stream) {
   if (plan.kind == kSmall) {
@@ -1272,13 +1294,14 @@ static int launch_main(const FusedArgs& a, const FusedPlan& plan, bool want_argm
     else if (plan.small_nbt == 1) TOME_SMALL(1, 16);
     else TOME_SMALL(2, 16);
 #undef TOME_SMALL
-    return n >= 2 ? n : -1;
+    return n;  // >= 2: fused_plan only picks this kernel when it can be placed
   }
   if (plan.kind == kDma) {
     if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.grid, stream);
     else launch_dma<ENT, false>(a, plan.dma_nbt, plan.grid, stream);
   } else {
-    hipLaunchKernelGGL(fused_lmhead_kernel<ENT>, dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
+    if (want_argmax) hipLaunchKernelGGL((fused_lmhead_kernel<ENT, true>), dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
+    else hipLaunchKernelGGL((fused_lmhead_kernel<ENT, false>), dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
   }
   return 0;
 }
@@ -1301,14 +1324,9 @@ static hipError_t fused_launch_impl(const void* hidden, const void* hidden_ref, 
   if (row_valid) {
     n_valid = reinterpret_cast<int32_t*>(ws);
     row_index = reinterpret_cast<int32_t*>(ws + off_index());
-    CompactArgs c{row_valid, row_index, n_valid, out_lp, out_lse, out_entropy, out_ref_lp, out_argmax, (int)n_tokens,
-                  plan.bt, plan.slots, plan.n_vtiles};
+    CompactArgs c{row_valid, row_index, n_valid, out_lp, out_lse, out_entropy, out_ref_lp, out_k3, out_argmax,
+                  (int)n_tokens, plan.bt, plan.slots, plan.n_vtiles};
     hipLaunchKernelGGL(compact_rows_kernel, dim3(1), dim3(1024), 0, stream, c);
-    if (out_k3) {
-      CompactArgs c2{row_valid, row_index, n_valid, out_k3, nullptr, nullptr, nullptr, nullptr, (int)n_tokens,
-                     plan.bt, plan.slots, plan.n_vtiles};
-      hipLaunchKernelGGL(compact_rows_kernel, dim3(1), dim3(1024), 0, stream, c2);
-    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -1320,7 +1338,7 @@ static hipError_t fused_launch_impl(const void* hidden, const void* hidden_ref, 
   a.n_valid = n_valid;
   a.hidden_stride_b = (uint32_t)(hidden_stride * 2);
   a.weight_stride_b = (uint32_t)(weight_stride * 2);
-  a.hidden_bytes = (uint32_t)(((n_tokens - 1) * hidden_stride + H) * 2);
+  a.hidden_bytes = (uint32_t)(((n_tokens - 1) * hidden_stride + H) * 2);  // read by the generic kernel only (< 4 GiB there)
   const char* second_hidden = static_cast<const char*>(hidden_ref);
   if (norm_weight) {  // normalise the valid rows into a dense buffer and multiply that
     char* normed = ws + off_partials(n_tokens) + (second ? 2 : 1) * partial_bytes(n_tokens, H, V);
@@ -1356,7 +1374,6 @@ static hipError_t fused_launch_impl(const void* hidden, const void* hidden_ref, 
   a.partials = p0;
   int n_parts = out_entropy ? launch_main<true>(a, plan, out_argmax != nullptr, stream)
                             : launch_main<false>(a, plan, out_argmax != nullptr, stream);
-  if (n_parts < 0) return hipErrorLaunchFailure;
   if (n_parts > 0) {  // small-batch kernel: one part per workgroup, whatever the mask
     a.sched = FusedSchedule{1, n_parts / kPartsPerSplit, n_parts, 0};
     a.sched_dev = nullptr;
@@ -1366,7 +1383,7 @@ static hipError_t fused_launch_impl(const void* hidden, const void* hidden_ref, 
     a.weight = static_cast<const char*>(w1);
     a.hidden = second_hidden;
     a.partials = p1;
-    if (launch_main<false>(a, plan, false, stream) < 0) return hipErrorLaunchFailure;
+    launch_main<false>(a, plan, false, stream);
     a.hidden = first_hidden;
   }
   hipError_t e = hipGetLastError();
@@ -1383,13 +1400,6 @@ static hipError_t fused_launch_impl(const void* hidden, const void* hidden_ref, 
   c.out_ref_lp = out_ref_lp;
   c.out_k3 = out_k3;
   c.out_argmax = out_argmax;
-  c.hidden = a.hidden;
-  c.hidden_index = a.hidden_index;
-  c.weight = static_cast<const char*>(w0);
-  c.hidden_stride_b = a.hidden_stride_b;
-  c.weight_stride_b = a.weight_stride_b;
-  c.H = a.H;
-  c.V = a.V;
   c.n_tokens = (int)n_tokens;
   c.sched_dev = a.sched_dev;
   c.sched = a.sched;

@@ -247,9 +247,10 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
 
   const bool big_range = (u1 - u0) * kVec + n_tail > kSampCap;
   if (tid == 0) sh.cnt = 0;  // published by the first barrier below, before any candidate is offered
-  // A candidate: an element at or above the bound (value first, then the whole key).
+  // A candidate: a logit above -inf (a -inf logit has probability zero and is never drawn; NaN fails every
+  // compare) at or above the bound (value first, then the whole key).
   auto offer = [&](float x, int64_t idx, uint64_t thr, float thr_val) {
-    if (x >= thr_val) {
+    if (x >= thr_val && x > -INFINITY) {
       const uint64_t key = make_key(x, (uint32_t)idx);
       if (key >= thr) {
         const int pos = atomicAdd(&sh.cnt, 1);
@@ -355,30 +356,8 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
       absorb<1, false, true>(st, x, (int)u, a.scale);
     }
   }
-  // This lane's maximum as a key: the first element of unit st.bi that equals st.mx.
-  uint64_t lane_key = 0;
-  if (st.bi != 0x7fffffff) {
-    int64_t idx = -1;
-    if constexpr (CACHED) {  // the unit is still in registers
-#pragma unroll
-      for (int q = kSampCached - 1; q >= 0; --q)
-        if (st.bi == (int)(u0 + tid + q * kRowWG)) {
-          float x[kVec];
-          Elem<T>::unpack(cached[q], x);
-#pragma unroll
-          for (int i = kVec - 1; i >= 0; --i)
-            if (x[i] == st.mx) idx = (int64_t)st.bi * kVec + i;
-        }
-    }
-    if (idx < 0) {  // a tail element, or the streaming variants: read the unit again
-      const int64_t first = st.bi < n_units ? (int64_t)st.bi * kVec : n_units * kVec + (st.bi - n_units);
-      const int count = st.bi < n_units ? kVec : 1;
-      idx = first;
-      for (int i = count - 1; i >= 0; --i)
-        if (Elem<T>::load1(row + first + i) == st.mx) idx = first + i;
-    }
-    lane_key = make_key(st.mx, (uint32_t)idx);
-  }
+  // This lane's maximum, or -inf when it saw nothing above the floor.
+  const float lane_max = st.bi != 0x7fffffff ? st.mx : -INFINITY;
   const RowStat tot = block_reduce(st, a.scale, sh.red);  // valid in wave 0; its barrier also ends the offers of pass 1
 
   int m = 0;
@@ -396,7 +375,7 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
 
   // ---- theta: k-th largest lane maximum (ranges that fit the buffer skip the bound) --------------
   uint64_t theta = 0;
-  if (scan && big_range) theta = bound_from_lane_maxima(sh, lane_key != 0 ? st.mx : -INFINITY, k);
+  if (scan && big_range) theta = bound_from_lane_maxima(sh, lane_max, k);
   else if (scan && collected) __syncthreads();
 
   // ---- pass 2: collect every element >= theta ---------------------------------------------------
