@@ -263,27 +263,69 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
   // ---- pass 1: full-vocabulary statistics and this lane's own maximum --------------------------
   RowStat st = stat_identity();
   u32x4 cached[CACHED ? kSampCached : 1];
+  float lane_max = -INFINITY;  // this lane's largest element, or -inf when it saw nothing above -inf
+  RowStat tot = stat_identity();
+  uint64_t theta = 0;
   if constexpr (CACHED) {
+    // Everything a lane owns is in registers, so the statistics take two sweeps over them instead of an online
+    // update: the maxima first, then the sum of 2^(y - m) against one reference per wave (no rescaling chain).
     const u32x4* p = reinterpret_cast<const u32x4*>(row);
 #pragma unroll
     for (int q = 0; q < kSampCached; ++q) {  // unconditional (clamped) loads: all eight in flight together
       const int64_t u = u0 + tid + q * kRowWG;
       cached[q] = p[u < u1 ? u : 0];         // unit 0 exists (checked on the host)
     }
+    float tail[Elem<T>::kVec - 1];           // single elements after the last whole unit: lane 0 of the last split
+#pragma unroll
+    for (int e = 0; e < kVec - 1; ++e) tail[e] = (tid == 0 && e < n_tail) ? Elem<T>::load1(row + n_units * kVec + e) : -INFINITY;
 #pragma unroll
     for (int q = 0; q < kSampCached; ++q)
       if (u0 + tid + q * kRowWG < u1) {
         float x[kVec];
         Elem<T>::unpack(cached[q], x);
-        absorb<kVec, false, true>(st, x, (int)(u0 + tid + q * kRowWG), a.scale);
-        __builtin_amdgcn_sched_barrier(0);  // one unit at a time: hoisting all eight overflows the registers
+        lane_max = fmaxf(lane_max, max_of<kVec>(x));
       }
-    if (tid == 0) {
-      for (int e = 0; e < n_tail; ++e) {
-        float x[1] = {Elem<T>::load1(row + n_units * kVec + e)};
-        absorb<1, false, true>(st, x, (int)(n_units + e), a.scale);
+#pragma unroll
+    for (int e = 0; e < kVec - 1; ++e) lane_max = fmaxf(lane_max, tail[e]);
+    float wmax = lane_max;  // maximum of the wave
+    wmax = fmaxf(wmax, wave_exchange<0>(wmax));
+    wmax = fmaxf(wmax, wave_exchange<1>(wmax));
+    wmax = fmaxf(wmax, wave_exchange<2>(wmax));
+    wmax = fmaxf(wmax, wave_exchange<3>(wmax));
+    wmax = fmaxf(wmax, wave_exchange<4>(wmax));
+    wmax = fmaxf(wmax, wave_exchange<5>(wmax));
+    const float mref = fmaxf(wmax, kMaxFloor);
+    const float mm = mref * a.scale;
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int q = 0; q < kSampCached; ++q)
+      if (u0 + tid + q * kRowWG < u1) {
+        float x[kVec];
+        Elem<T>::unpack(cached[q], x);
+#pragma unroll
+        for (int i = 0; i < kVec; i += 2) {
+          s0 += fast_exp2(fmaf(x[i], a.scale, -mm));
+          s1 += fast_exp2(fmaf(x[i + 1], a.scale, -mm));
+        }
       }
+#pragma unroll
+    for (int e = 0; e < kVec - 1; ++e) s0 += fast_exp2(fmaf(tail[e], a.scale, -mm));  // -inf adds nothing
+    float ws = s0 + s1;
+    ws += wave_exchange<0>(ws);
+    ws += wave_exchange<1>(ws);
+    ws += wave_exchange<2>(ws);
+    ws += wave_exchange<3>(ws);
+    ws += wave_exchange<4>(ws);
+    ws += wave_exchange<5>(ws);
+    if (lane == 0) {
+      sh.red.mx[wave] = mref;
+      sh.red.s[wave] = ws;
     }
+    __syncthreads();  // also publishes sh.cnt == 0
+#pragma unroll
+    for (int w = 0; w < kRowWaves; ++w) stat_merge(tot, RowStat{sh.red.mx[w], sh.red.s[w], 0.f, 0x7fffffff}, a.scale);
+    // theta: k-th largest lane maximum (ranges that fit the buffer skip the bound)
+    if (big_range) theta = bound_from_lane_maxima(sh, lane_max, k);
   } else if constexpr (VECTOR) {
     // Streaming variant: candidates are collected during this one pass.  The k-th largest of the
     // lanes' maxima over their FIRST units is already a lower bound of the row's k-th largest, so
@@ -356,27 +398,25 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
       absorb<1, false, true>(st, x, (int)u, a.scale);
     }
   }
-  // This lane's maximum, or -inf when it saw nothing above the floor.
-  const float lane_max = st.bi != 0x7fffffff ? st.mx : -INFINITY;
-  const RowStat tot = block_reduce(st, a.scale, sh.red);  // valid in wave 0; its barrier also ends the offers of pass 1
-
   int m = 0;
   bool scan = true;
-  if (collected) {
-    const int offered = sh.cnt;
-    if (offered <= kSampCap) {
-      m = offered;
-      scan = false;
-    } else {  // the early bound let too much through: fall back to the bound from the whole range and rescan
-      __syncthreads();
-      if (tid == 0) sh.cnt = 0;
+  if constexpr (!CACHED) {
+    lane_max = st.bi != 0x7fffffff ? st.mx : -INFINITY;  // nothing above the floor seen: -inf
+    tot = block_reduce(st, a.scale, sh.red);  // valid in wave 0; its barrier also ends the offers of pass 1
+    if (collected) {
+      const int offered = sh.cnt;
+      if (offered <= kSampCap) {
+        m = offered;
+        scan = false;
+      } else {  // the early bound let too much through: fall back to the bound from the whole range and rescan
+        __syncthreads();
+        if (tid == 0) sh.cnt = 0;
+      }
     }
+    // ---- theta: k-th largest lane maximum (ranges that fit the buffer skip the bound) --------------
+    if (scan && big_range) theta = bound_from_lane_maxima(sh, lane_max, k);
+    else if (scan && collected) __syncthreads();
   }
-
-  // ---- theta: k-th largest lane maximum (ranges that fit the buffer skip the bound) --------------
-  uint64_t theta = 0;
-  if (scan && big_range) theta = bound_from_lane_maxima(sh, lane_max, k);
-  else if (scan && collected) __syncthreads();
 
   // ---- pass 2: collect every element >= theta ---------------------------------------------------
   // sh.cnt is zero here: cleared before the first barrier, and again after an overflow.
