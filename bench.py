@@ -37,7 +37,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 SETTLE_MS = 60.0                # untimed GPU-busy time in front of every timed region (default of --settle-ms)
 SETTLE = {"ms": SETTLE_MS}
 SETTLE_MAX_LAUNCHES = 2000
-LEGS = ["row", "config1", "ceiling", "fused", "config4", "config5", "small", "midsize", "decode", "lora"]
+LEGS = ["row", "config1", "ceiling", "fused", "gemm", "config4", "config5", "small", "midsize", "decode", "lora"]
 SUSTAINED = {"tflops": None}    # bf16 MFMA rate of the probe loop on random operands, measured by the `ceiling` leg
 
 
@@ -177,9 +177,25 @@ def bench_row(dev, steps, warmup, variant="both"):
     assert torch.isfinite(got).all() and (got <= 1e-5).all()
     assert (got[valid == 0] == 0).all()
 
+    # the same rows as a packed row list (tome_row_logprob_rows): only the valid rows are launched
+    idx = torch.nonzero(valid).view(-1).to(torch.int32).contiguous()
+    tg_packed = tg[idx.long()].contiguous()
+    lp_packed = torch.empty(n_valid, dtype=torch.float32, device=dev)
+    ws2_bytes = lib.tome_row_logprob_workspace(n_valid, V)
+    ws2 = torch.empty(max(ws2_bytes, 1), dtype=torch.uint8, device=dev)
+
+    def step_list():
+        _lib.check(lib.tome_row_logprob_rows(flat.data_ptr(), 1, rows, V, V, idx.data_ptr(), n_valid, tg_packed.data_ptr(), 1.0,
+                                             lp_packed.data_ptr(), None, None, None, ws2.data_ptr(), ws2_bytes, stream))
+    step_list()
+    torch.cuda.synchronize()
+    assert torch.equal(lp_packed, got[idx.long()])       # the row list scores exactly what the mask scores
+
     out = {"n_valid": n_valid, "rows": rows, "bytes_mask": n_valid * V * 2, "bytes_all": rows * V * 2}
     if variant in ("both", "mask"):
         out["mask"] = time_steps(lambda: step(True), steps, warmup)
+    if variant in ("both", "list"):
+        out["list"] = time_steps(step_list, steps, warmup)
     if variant in ("both", "all"):
         out["all"] = time_steps(lambda: step(False), steps, warmup)
     del logits, flat
@@ -260,6 +276,25 @@ def bench_fused(dev, steps, warmup, n=4096, H=1024, temperature=1.0, lengths=Non
     tm = time_steps(step, steps, warmup)
     tm.update({"tokens": n, "valid": n_valid, "H": H, "flop": 2.0 * n_valid * H * V,
                "bytes": V * H * 2 + n_valid * H * 2})
+    return tm
+
+
+def bench_library_gemm(dev, steps, warmup, n=4096, H=1024):
+    """The vendor library's bf16 GEMM alone on config 3's shape, for scale: logits = hidden @ W^T written as bf16
+    [n, V] (what mlx-impl/model.py:538 materialises), no softmax.  torch.mm dispatches to hipBLASLt / rocBLAS."""
+    import torch
+    g = torch.Generator(device=dev).manual_seed(4321)
+    hidden = torch.randn((n, H), device=dev, generator=g).to(torch.bfloat16)
+    weight = (torch.randn((V, H), device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    out = torch.empty((n, V), device=dev, dtype=torch.bfloat16)
+    wt = weight.t()
+
+    def step():
+        torch.mm(hidden, wt, out=out)
+    step()
+    torch.cuda.synchronize()
+    tm = time_steps(step, steps, warmup)
+    tm.update({"tokens": n, "H": H, "flop": 2.0 * n * H * V})
     return tm
 
 
@@ -465,8 +500,9 @@ def main():
                     help="untimed GPU-busy time in front of every timed region (counter runs pass 0)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None, help="comma-separated subset of: " + ", ".join(LEGS))
-    ap.add_argument("--row-variant", choices=["both", "mask", "all"], default="both",
-                    help="time config 2 with its padding mask, without it, or both (profiling runs pick one)")
+    ap.add_argument("--row-variant", choices=["both", "mask", "list", "all"], default="both",
+                    help="time config 2 with its padding mask, with the valid rows as a packed list, without the mask, "
+                         "or all three (profiling runs pick one)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so a counter run can scale FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -519,6 +555,17 @@ def main():
                 "roofline": hbm_roofline(row["bytes_mask"], t["ms"], traffic_of("row_logprob_config2_masked"),
                                          "row_logprob_kernel<bf16>")}
             done("headline")
+        if "list" in row:
+            t = row["list"]
+            legs["row_list"] = {
+                "value": row["n_valid"] / (t["ms"] * 1e-3), "unit": "token-logprobs/s", **timing_fields(t),
+                "dtype": "f32", "input_dtype": "bf16",
+                "config": {"workload": "config 2 with the valid rows given as a packed row list instead of a mask "
+                                       "(tome_row_logprob_rows): bf16 logits [8x512, 151936], lengths~U[64,512], packed fp32 out",
+                           "rows": row["rows"], "valid_rows": row["n_valid"], "vocab": V, "temperature": 1.0},
+                "roofline": hbm_roofline(row["bytes_mask"], t["ms"], traffic_of("row_logprob_config2_masked"),
+                                         "row_logprob_kernel<bf16>")}
+            done("row_list")
         if "all" in row:
             t = row["all"]
             legs["all_rows"] = {
@@ -562,6 +609,14 @@ def main():
                        "tokens": t["tokens"], "hidden": t["H"], "vocab": V, "temperature": 1.0},
             "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("fused_lmhead_config3"), "fused_lmhead_dma_kernel")}
         done("fused_lmhead")
+    if "gemm" in only:
+        t = bench_library_gemm(dev, K, W)
+        legs["library_gemm_config3"] = {
+            "value": t["flop"] / (t["ms"] * 1e-3) / 1e12, "unit": "TFLOP/s", **timing_fields(t), "dtype": "bf16 x bf16 -> bf16",
+            "config": {"workload": "for scale, not part of the path: torch.mm (vendor GEMM library) on config 3's shape, bf16 logits "
+                                   "[4096, 151936] written, no softmax", "tokens": t["tokens"], "hidden": t["H"], "vocab": V},
+            "roofline": mfma_roofline(t["flop"], t["ms"], None, "vendor library GEMM (hipBLASLt / rocBLAS via torch.mm)")}
+        done("library_gemm_config3")
     if "config4" in only:
         t = bench_fused(dev, K, W, n=16 * 1024, H=2560, temperature=0.7, lengths=(16, 1024, 128, 1024), seed=444)
         legs["config4_fused_varlen"] = {

@@ -74,6 +74,22 @@ int tome_row_logprob(const void* logits, int dtype, int64_t rows, int64_t V, int
                      float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- Row kernel over a list of rows -----------------------------------------------
+ * The same kernel for the rows a caller names: problem i reads row row_index[i] of `logits`
+ * ([n_rows, V]) and owns targets[i] and out_*[i], so inputs and outputs are PACKED in list order.
+ * It replaces the reference's slicing of the completion rows out of the padded batch,
+ *   chunk_logits[b, p_len - 1 : p_len - 1 + len(c_toks), :]          mlx-impl/node.py:449
+ * followed by local_compute_logprobs on the slice (node.py:400-404, 451), for all sequences of a
+ * chunk in one launch: prompt and padding rows are neither read nor launched, and the packed
+ * result is what Completion.ref_log_probs takes (node.py:457-458).  `row_index` is a device
+ * array; an entry outside [0, n_rows) is not read and scores NaN (argmax -1).  Workspace:
+ * tome_row_logprob_workspace(n_index, V).
+ */
+int tome_row_logprob_rows(const void* logits, int dtype, int64_t n_rows, int64_t V, int64_t row_stride,
+                          const int32_t* row_index, int64_t n_index, const int32_t* targets,
+                          float temperature, float* out_lp, float* out_lse, float* out_entropy,
+                          int32_t* out_argmax, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- Row kernel for callers that cannot allocate ------------------------------------
  * No counterpart in the reference.  It exists for callers that cannot hand over a workspace
  * because they cannot allocate one: code running under HIP graph capture, serving loops with

@@ -80,6 +80,13 @@ def test_argument_checks_run_on_host():
     assert na(dtype=7) == -2 and na(V=0) == -3 and na(stride=63) == -3 and na(T=0.0) == -5
     assert na(logits=None) == -1 and na(targets=None) == -1 and na(lp=None) == -1 and na(rows=0) == 0
     assert na(logits=P + 1) == -6
+    rl = lambda **k: lib.tome_row_logprob_rows(k.get("logits", P), k.get("dtype", 1), k.get("rows", 4), k.get("V", 64),
+                                               k.get("stride", 64), k.get("idx", P), k.get("n", 3), k.get("targets", P),
+                                               k.get("T", 1.0), k.get("lp", P), None, None, None, None, 0, None)
+    assert rl(dtype=7) == -2 and rl(V=0) == -3 and rl(stride=63) == -3 and rl(n=-1) == -3 and rl(rows=-1) == -3
+    assert rl(T=0.0) == -5 and rl(logits=None) == -1 and rl(idx=None) == -1 and rl(targets=None) == -1 and rl(lp=None) == -1
+    assert rl(n=0) == 0 and rl(logits=P + 1) == -6
+    assert rl(rows=4096, V=151936, stride=151936, n=64) == -4        # 64 listed rows are split: workspace needed
     fused = lambda **k: lib.tome_fused_lmhead_logprob(k.get("h", P), k.get("w", P), k.get("n", 8), k.get("H", 64),
                                                       k.get("V", 100), k.get("hs", 64), k.get("ws", 64), P, None,
                                                       k.get("T", 1.0), k.get("lp", P), None, None, None, None, 0, None)

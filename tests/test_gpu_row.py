@@ -209,3 +209,36 @@ def test_entry_points_replay_correctly_from_a_hip_graph(dev):
         for a, b in zip(got, [e_row.lp, e_row.argmax, e_fused.lp, e_fused.entropy]):
             assert torch.equal(a, b)
         (h.float() @ w.float().T).sum().item()                       # unrelated eager work between replays
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,V,n_index", [(64, 151936, 37), (700, 4097, 700), (4096, 8192, 1500), (9, 50, 30)])
+def test_row_list_matches_full_call_and_oracle(dev, dtype, rows, V, n_index):
+    """tome_row_logprob_rows (the completion rows of mlx-impl/node.py:449 as a packed list) against the oracle and
+    against the plain call on the gathered rows; order, repeats and out-of-range entries of the list are honoured."""
+    rng = np.random.default_rng(rows + V + n_index)
+    x = torch.from_numpy((rng.standard_normal((rows, V)) * 2.5).astype(np.float32)).to(dev).to(dtype)
+    idx = rng.integers(0, rows, size=n_index).astype(np.int32)       # unsorted, with repeats
+    idx[: min(rows, n_index)] = rng.permutation(rows)[: min(rows, n_index)]
+    t = rng.integers(0, V, size=n_index).astype(np.int32)
+    bad = [1, n_index - 1]
+    idx_bad = idx.copy()
+    idx_bad[bad[0]], idx_bad[bad[1]] = rows, -1                       # not rows of the matrix
+    got = tome_amd.token_logprobs_rows(x, torch.from_numpy(idx_bad).to(dev), torch.from_numpy(t).to(dev), 0.9,
+                                       want_lse=True, want_entropy=True, want_argmax=True)
+    ok = np.ones(n_index, bool)
+    ok[bad] = False
+    src = x.float().cpu().numpy() if dtype == torch.float32 else bf16_bits_of(x)
+    lp, lse, ent, am = (v.cpu().numpy() for v in got)
+    assert lp.shape == (n_index,)
+    np.testing.assert_allclose(lp[ok], oracle.logprob_rows(src[idx[ok]], t[ok], 0.9), atol=1e-4, rtol=0)
+    np.testing.assert_allclose(lse[ok], oracle.lse_rows(src[idx[ok]], 0.9), atol=1e-4, rtol=0)
+    np.testing.assert_allclose(ent[ok], oracle.entropy_rows(src[idx[ok]], 0.9), atol=1e-4, rtol=0)
+    np.testing.assert_array_equal(am[ok], oracle.argmax_rows(src[idx[ok]]))
+    assert np.isnan(lp[bad]).all() and np.isnan(lse[bad]).all() and (am[bad] == -1).all()
+    # against the plain entry point on the gathered rows (same number of problems -> same split of a row)
+    dense = tome_amd.token_logprobs(x[torch.from_numpy(idx[ok]).to(dev).long()], torch.from_numpy(t[ok]).to(dev), 0.9,
+                                    want_lse=True, want_argmax=True)
+    np.testing.assert_allclose(lp[ok], dense.lp.cpu().numpy(), atol=2e-6, rtol=0)
+    np.testing.assert_array_equal(am[ok], dense.argmax.cpu().numpy())
+

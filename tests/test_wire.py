@@ -26,6 +26,9 @@ def test_packed_chunks_reproduce_the_entry_bookkeeping(T, batch):
         assert int(chunk.valid.sum()) == chunk.n_scored
         logits = stub_logits(chunk.ids.astype(np.uint32))
         m = chunk.valid.astype(bool)
+        # the packed row list of the chunk names exactly the valid positions, in row-major order
+        assert np.array_equal(chunk.scored_rows, np.flatnonzero(m.reshape(-1))) and chunk.scored_rows.dtype == np.int32
+        assert np.array_equal(chunk.scored_targets, chunk.targets[m]) and len(chunk.scored_rows) == chunk.n_scored
         flat = oracle.local_compute_logprobs_f32(logits[m], chunk.targets[m].astype(np.uint32), T or 1.0)
         n_got += tome_amd.scatter_ref_logprobs(chunk, flat, results)
     assert n_got == n_want

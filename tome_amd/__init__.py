@@ -11,6 +11,7 @@ from .logprob import (  # noqa: F401
     fused_log_softmax,
     local_compute_logprobs,
     token_logprobs,
+    token_logprobs_rows,
     sample_tokens,
     DecodeStepGraph,
     fused_lmhead_logprobs,
@@ -29,7 +30,7 @@ from .wire import (  # noqa: F401
 from ._lib import TomeError, lib_path, load_library  # noqa: F401
 
 __all__ = [
-    "fused_log_softmax", "local_compute_logprobs", "token_logprobs", "sample_tokens", "DecodeStepGraph", "fused_lmhead_logprobs",
+    "fused_log_softmax", "local_compute_logprobs", "token_logprobs", "token_logprobs_rows", "sample_tokens", "DecodeStepGraph", "fused_lmhead_logprobs",
     "grpo_dual_logprobs", "grpo_pair_logprobs", "LayerUpdate", "WeightUpdateResponse", "WeightUpdateServicer",
     "apply_weight_update", "lora_merge", "TokenLogprobs", "SampledTokens", "DualLogprobs", "Prompt", "Completion", "PromptRollout",
     "RefLogprobServicer", "rollout_decode", "judge_decode", "PackedRefChunk", "pack_ref_work", "scatter_ref_logprobs",

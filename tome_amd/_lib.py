@@ -20,6 +20,8 @@ SIGNATURES = {
     "tome_row_logprob_workspace": (c_size_t, [c_int64, c_int64]),
     "tome_row_logprob": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "tome_row_logprob_rows": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_float,
+                                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "tome_row_logprob_noalloc": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "tome_row_sample_workspace": (c_size_t, [c_int, c_int64, c_int64, c_int]),

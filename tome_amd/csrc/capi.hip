@@ -11,6 +11,10 @@ hipError_t row_logprob_launch(const void* logits, int dtype, int64_t rows, int64
                               const int32_t* targets, const int32_t* row_valid, float temperature,
                               float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
                               void* workspace, hipStream_t stream);
+hipError_t row_logprob_launch_rows(const void* logits, int dtype, int64_t n_rows, const int32_t* row_index, int64_t rows,
+                                   int64_t V, int64_t row_stride, const int32_t* targets, const int32_t* row_valid,
+                                   float temperature, float* out_lp, float* out_lse, float* out_entropy,
+                                   int32_t* out_argmax, void* workspace, hipStream_t stream);
 int row_splits_for(int64_t rows, int64_t V, int vec);
 hipError_t row_logprob_noalloc_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
                                       const int32_t* targets, const int32_t* row_valid, float temperature,
@@ -115,6 +119,25 @@ int tome_row_logprob(const void* logits, int dtype, int64_t rows, int64_t V, int
   return hip_result(tome::row_logprob_launch(logits, dtype, rows, V, row_stride, targets, row_valid, temperature,
                                              out_lp, out_lse, out_entropy, out_argmax, workspace,
                                              static_cast<hipStream_t>(stream)));
+}
+
+int tome_row_logprob_rows(const void* logits, int dtype, int64_t n_rows, int64_t V, int64_t row_stride,
+                          const int32_t* row_index, int64_t n_index, const int32_t* targets, float temperature,
+                          float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+  if (dtype != TOME_F32 && dtype != TOME_BF16) return TOME_E_DTYPE;
+  if (bad_matrix(n_rows, V, row_stride) || bad_matrix(n_index, V, row_stride)) return TOME_E_SHAPE;
+  if (bad_temperature(temperature)) return TOME_E_TEMPERATURE;
+  if (n_index == 0) return TOME_OK;
+  if (!logits || !row_index) return TOME_E_NULL;
+  if (out_lp && !targets) return TOME_E_NULL;
+  if (!out_lp && !out_lse && !out_entropy && !out_argmax) return TOME_E_NULL;
+  const size_t need = tome_row_logprob_workspace(n_index, V);
+  if (need > 0 && (!workspace || workspace_bytes < need)) return TOME_E_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(logits) % (dtype == TOME_F32 ? 4 : 2) != 0) return TOME_E_ALIGN;
+  return hip_result(tome::row_logprob_launch_rows(logits, dtype, n_rows, row_index, n_index, V, row_stride, targets,
+                                                  nullptr, temperature, out_lp, out_lse, out_entropy, out_argmax,
+                                                  workspace, static_cast<hipStream_t>(stream)));
 }
 
 int tome_row_logprob_noalloc(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,

@@ -22,8 +22,12 @@ struct RowPartial {  // one per (row, split) in the workspace
   int bi;
 };
 
+// A launch scores `problems`: problem i reads row i of the logits - or, with a row list, row row_index[i] - and
+// owns entry i of targets, row_valid, the outputs and the partials.
 struct RowArgs {
   const void* logits;
+  const int32_t* row_index;  // nullable: problem -> row of `logits` (a row outside [0, n_rows) scores NaN, argmax -1)
+  int64_t n_rows;            // rows the logits matrix holds (only read with a row list)
   const int32_t* targets;
   const int32_t* row_valid;
   float* out_lp;
@@ -78,7 +82,7 @@ template <typename T, bool VECTOR, bool ENT, bool AMAX>
 __global__ __launch_bounds__(kRowWG) void row_logprob_kernel(RowArgs a) {
   constexpr int kVec = VECTOR ? Elem<T>::kVec : 1;
   __shared__ RowLds lds;
-  const int64_t r = blockIdx.x / a.splits;
+  const int64_t r = blockIdx.x / a.splits;  // problem index
   const int split = blockIdx.x % a.splits;
   const int tid = threadIdx.x;
 
@@ -91,8 +95,18 @@ __global__ __launch_bounds__(kRowWG) void row_logprob_kernel(RowArgs a) {
     }
     return;
   }
+  const int64_t src = a.row_index ? (int64_t)a.row_index[r] : r;  // row of the logits matrix
+  if (a.row_index && (uint64_t)src >= (uint64_t)a.n_rows) {        // a list entry that names no row: not read
+    if (split == 0 && tid == 0) {
+      if (a.out_lp) a.out_lp[r] = __builtin_nanf("");
+      if (a.out_lse) a.out_lse[r] = __builtin_nanf("");
+      if (ENT) a.out_entropy[r] = __builtin_nanf("");
+      if (AMAX) a.out_argmax[r] = -1;
+    }
+    return;
+  }
 
-  const T* row = static_cast<const T*>(a.logits) + r * a.row_stride;
+  const T* row = static_cast<const T*>(a.logits) + src * a.row_stride;
   const int64_t n_units = a.V / kVec;
   const int64_t per_split = (n_units + a.splits - 1) / a.splits;
   const int64_t u0 = per_split * split;
@@ -164,8 +178,10 @@ template <typename T, bool VECTOR, bool ENT, bool AMAX>
 __global__ __launch_bounds__(64) void row_combine_kernel(RowArgs a) {
   const int64_t r = blockIdx.x;
   if (a.row_valid && a.row_valid[r] == 0) return;  // outputs already zeroed by the main kernel
+  const int64_t src = a.row_index ? (int64_t)a.row_index[r] : r;
+  if (a.row_index && (uint64_t)src >= (uint64_t)a.n_rows) return;  // outputs already written by the main kernel
   const int lane = threadIdx.x;
-  const T* row = static_cast<const T*>(a.logits) + r * a.row_stride;
+  const T* row = static_cast<const T*>(a.logits) + src * a.row_stride;
   float x_t = 0.f;
   if (lane == 0) x_t = load_target_logit<T>(a, row, r);
   RowStat st = stat_identity();
@@ -221,15 +237,19 @@ int row_splits_for(int64_t rows, int64_t V, int vec) {
   return (int)s;
 }
 
-hipError_t row_logprob_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
-                              const int32_t* targets, const int32_t* row_valid, float temperature,
-                              float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
-                              void* workspace, hipStream_t stream) {
+// `rows` problems.  With `row_index` (device, one entry per problem) problem i reads row row_index[i] of a matrix
+// of `n_rows` rows; without it, row i.
+hipError_t row_logprob_launch_rows(const void* logits, int dtype, int64_t n_rows, const int32_t* row_index, int64_t rows,
+                                   int64_t V, int64_t row_stride, const int32_t* targets, const int32_t* row_valid,
+                                   float temperature, float* out_lp, float* out_lse, float* out_entropy,
+                                   int32_t* out_argmax, void* workspace, hipStream_t stream) {
   const int esize = dtype == 0 ? 4 : 2;
   const int vec = 16 / esize;
   const bool vector_ok = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && (row_stride % vec == 0);
   RowArgs a;
   a.logits = logits;
+  a.row_index = row_index;
+  a.n_rows = n_rows;
   a.targets = targets;
   a.row_valid = row_valid;
   a.out_lp = out_lp;
@@ -246,6 +266,14 @@ hipError_t row_logprob_launch(const void* logits, int dtype, int64_t rows, int64
   }
   return vector_ok ? dispatch_flags<uint16_t, true>(a, rows, stream)
                    : dispatch_flags<uint16_t, false>(a, rows, stream);
+}
+
+hipError_t row_logprob_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                              const int32_t* targets, const int32_t* row_valid, float temperature,
+                              float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
+                              void* workspace, hipStream_t stream) {
+  return row_logprob_launch_rows(logits, dtype, rows, nullptr, rows, V, row_stride, targets, row_valid, temperature,
+                                 out_lp, out_lse, out_entropy, out_argmax, workspace, stream);
 }
 
 // ---- allocation-free variant ---------------------------------------------------------------------

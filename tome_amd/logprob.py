@@ -190,6 +190,38 @@ def token_logprobs(logits: torch.Tensor, targets, temperature: float = 1.0, leng
     return TokenLogprobs(_shaped(lp), _shaped(lse), _shaped(ent), _shaped(amax))
 
 
+def token_logprobs_rows(logits: torch.Tensor, row_index, targets, temperature: float = 1.0, *,
+                        want_lse: bool = False, want_entropy: bool = False, want_argmax: bool = False) -> TokenLogprobs:
+    """``token_logprobs`` for a list of rows, packed: entry i scores row ``row_index[i]`` of the flattened
+    ``logits`` ([..., V] -> [rows, V]) against ``targets[i]``; every output has ``len(row_index)`` entries.
+
+    This is the slicing of mlx-impl/node.py:449 (the completion rows of each sequence of a padded chunk) and
+    local_compute_logprobs on the slices (node.py:400-404) for the whole chunk in one launch; rows that are not
+    listed are neither read nor launched.  An index outside the matrix scores NaN (argmax -1).
+    """
+    lib = _lib.load_library()
+    dev = _require_gpu(logits)
+    temperature = _check_temperature(temperature)
+    dtype = _dtype_code(logits)
+    x = _rows_view(logits)
+    rows, V = x.shape
+    idx = torch.as_tensor(row_index, device=dev) if not isinstance(row_index, torch.Tensor) else row_index
+    n = idx.numel()
+    idx = _as_i32(idx, n, dev, "row_index")
+    tg = _as_i32(targets, n, dev, "targets")
+    with _on_device(dev):
+        lp = torch.empty(n, dtype=torch.float32, device=dev)
+        lse = torch.empty(n, dtype=torch.float32, device=dev) if want_lse else None
+        ent = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
+        amax = torch.empty(n, dtype=torch.int32, device=dev) if want_argmax else None
+        ws_bytes = lib.tome_row_logprob_workspace(n, V)
+        ws = _workspace(ws_bytes, dev)
+        _lib.check(lib.tome_row_logprob_rows(x.data_ptr(), dtype, rows, V, x.stride(0) if rows > 1 else V, idx.data_ptr(), n,
+                                             tg.data_ptr(), temperature, lp.data_ptr(), _ptr(lse), _ptr(ent), _ptr(amax),
+                                             _ptr(ws), ws_bytes, _stream(dev)))
+    return TokenLogprobs(lp, lse, ent, amax)
+
+
 def sample_tokens(logits: torch.Tensor, temperature: float, top_k: int = 20, *, uniforms=None,
                   generator: Optional[torch.Generator] = None, row_valid=None, lengths=None,
                   want_topk: bool = False) -> SampledTokens:

@@ -18,7 +18,7 @@ import numpy as np
 import torch
 
 from .wire import pack_ref_work, scatter_ref_logprobs
-from .logprob import fused_lmhead_logprobs, token_logprobs
+from .logprob import fused_lmhead_logprobs, token_logprobs_rows
 
 logger = logging.getLogger(__name__)
 
@@ -90,16 +90,18 @@ class RefLogprobServicer:
                 continue
             full_ids = torch.from_numpy(chunk.ids).to(self.device)
             out, _ = self.reference_model(full_ids, cache=None)           # node.py:443
-            tg = torch.from_numpy(chunk.targets).to(self.device)
-            rv = torch.from_numpy(chunk.valid).to(self.device)
+            # The scored positions - rows p_len-1 .. p_len-2+len(c) of each sequence (node.py:449) - packed in
+            # row-major order; one sync + one copy per chunk (node.py:456), of those positions only.
             if self.lm_head_weight is None:
-                lps = token_logprobs(out, tg, temp, row_valid=rv).lp
+                rows = torch.from_numpy(chunk.scored_rows).to(self.device)
+                tg = torch.from_numpy(chunk.scored_targets).to(self.device)
+                flat = token_logprobs_rows(out, rows, tg, temp).lp.cpu().numpy()   # only the listed rows are launched
             else:
+                tg = torch.from_numpy(chunk.targets).to(self.device)
+                rv = torch.from_numpy(chunk.valid).to(self.device)
                 lps = fused_lmhead_logprobs(out, self.lm_head_weight, tg, temp, row_valid=rv,
                                             norm_weight=self.final_norm_weight, norm_eps=self.norm_eps).lp
-            # one sync + one copy per chunk (node.py:456), of the scored positions only: rows
-            # p_len-1 .. p_len-2+len(c) of each sequence (node.py:449), packed in row-major order
-            flat = lps[rv.bool()].cpu().numpy()
+                flat = lps[rv.bool()].cpu().numpy()
             num_toks += scatter_ref_logprobs(chunk, flat, results)        # node.py:457-458
 
         elapsed = time.perf_counter() - t0

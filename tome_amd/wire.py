@@ -36,6 +36,16 @@ class PackedRefChunk:
     def n_scored(self) -> int:
         return int(self.cu_lens[-1])
 
+    @property
+    def scored_rows(self) -> np.ndarray:
+        """Rows of the flattened [B * max_len] batch that are scored, ascending (int32): the packed row list."""
+        return np.flatnonzero(self.valid.reshape(-1)).astype(np.int32)
+
+    @property
+    def scored_targets(self) -> np.ndarray:
+        """The targets of ``scored_rows``, in the same order (int32 [n_scored])."""
+        return self.targets.reshape(-1)[self.scored_rows]
+
 
 def pack_ref_work(prompts: Sequence, results: Sequence, G: int, max_ref_batch_size: int = 32) -> List[PackedRefChunk]:
     """The work list and chunking of mlx-impl/node.py:409-441 as packed arrays, one entry per chunk."""
