@@ -651,14 +651,14 @@ def main():
         mid = {}
         for n, H in ((160, 1024), (256, 1024), (64, 4096), (128, 4096)):
             t = bench_fused(dev, K, W, n=n, H=H, seed=1000 + n + H)
-            mid[f"{n}x{H}"] = {"ms_per_step": t["ms"], "median_ms": t["median_ms"],
+            mid[f"{n}x{H}"] = {**timing_fields(t),
                                "roofline": hbm_roofline(t["bytes"], t["ms"], None, "fused lm_head sweep + combine")}
             log(f"midsize {n}x{H}: {t['ms'] * 1e3:.1f} us, {mid[f'{n}x{H}']['roofline']['frac']:.3f} of HBM peak")
             torch.cuda.empty_cache()
         worst = min(mid.values(), key=lambda d: d["roofline"]["frac"])
         legs["fused_lmhead_small_batches"] = {
-            "value": worst["roofline"]["achieved"], "unit": "GB/s (lowest of the shapes)", "ms_per_step": worst["ms_per_step"],
-            "median_ms": worst["median_ms"], "min_ms": worst["median_ms"], "settle_launches": None,
+            "value": worst["roofline"]["achieved"], "unit": "GB/s (lowest of the shapes)",
+            **{k: worst[k] for k in ("ms_per_step", "median_ms", "min_ms", "settle_launches")},
             "dtype": "bf16 x bf16 -> f32",
             "config": {"workload": "fused lm_head + log-softmax where W streams once: tokens x hidden in {160x1024, 256x1024, "
                                    "64x4096, 128x4096}, V = 151936", "shapes": mid},
