@@ -959,40 +959,66 @@ struct CompactArgs {
   int bt, slots, n_vtiles;  // inputs of the schedule, which this kernel derives from n_valid
 };
 
+// Rows are taken in batches of up to 16384: each of the 16 waves owns a run of consecutive rows of a batch (a
+// sixteenth of the rows, at most 1024) and reads their mask values with 16 independent coalesced loads (lane
+// l of chunk c reads row first + 64 c + l), which stay in registers for the second sweep; counts come from ballots,
+// the waves' offsets from a scan through LDS.
 __global__ __launch_bounds__(1024) void compact_rows_kernel(CompactArgs a) {
+  constexpr int kChunks = 16;                       // 64-row chunks per wave and batch, at most
   __shared__ int wave_tot[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int per = (a.n + 1023) / 1024;
-  const int r0 = tid * per, r1 = min(a.n, r0 + per);
-  int cnt = 0;
-  for (int r = r0; r < r1; ++r) cnt += a.row_valid[r] != 0;
-  int inc = cnt;  // inclusive scan inside the wave
+  const uint64_t below = (1ull << lane) - 1;        // lanes in front of this one
+  int n_chunks = (int)((((int64_t)a.n + 15) / 16 + 63) / 64);  // per wave, so that small batches use all 16 waves
+  n_chunks = n_chunks > kChunks ? kChunks : n_chunks;
+  const int wave_rows = n_chunks * 64;
+  const int64_t batch_rows = 16 * (int64_t)wave_rows;
+  float* outs[5] = {a.out0, a.out1, a.out2, a.out3, a.out4};  // the float outputs that exist, packed to the front
+  int n_outs = 0;
 #pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const int up = __shfl_up(inc, off, 64);
-    if (lane >= off) inc += up;
-  }
-  if (lane == 63) wave_tot[wave] = inc;
-  __syncthreads();
-  int base = 0;
-  for (int w = 0; w < wave; ++w) base += wave_tot[w];
-  int pos = base + inc - cnt;
-  for (int r = r0; r < r1; ++r) {
-    if (a.row_valid[r] != 0) {
-      a.row_index[pos++] = r;
-    } else {
-      if (a.out0) a.out0[r] = 0.f;
-      if (a.out1) a.out1[r] = 0.f;
-      if (a.out2) a.out2[r] = 0.f;
-      if (a.out3) a.out3[r] = 0.f;
-      if (a.out4) a.out4[r] = 0.f;
-      if (a.out_argmax) a.out_argmax[r] = -1;
+  for (int o = 0; o < 5; ++o)
+    if (outs[o]) outs[n_outs++] = outs[o];
+  int done = 0;                                     // valid rows of earlier batches
+  for (int64_t b0 = 0; b0 < a.n; b0 += batch_rows) {
+    const int64_t first = b0 + (int64_t)wave * wave_rows;
+    int v[kChunks];
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c) {  // unconditional (clamped) loads: all of them in flight together
+      const int64_t r = first + c * 64 + lane;
+      v[c] = a.row_valid[r < a.n ? r : a.n - 1];
     }
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c) v[c] = (c < n_chunks && first + c * 64 + lane < a.n) ? v[c] : 0;
+    int cnt = 0;
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c) cnt += __builtin_popcountll(__ballot(v[c] != 0));
+    if (lane == 0) wave_tot[wave] = cnt;
+    __syncthreads();
+    int pos = done, total = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      pos += w < wave ? wave_tot[w] : 0;
+      total += wave_tot[w];
+    }
+    __syncthreads();                                // wave_tot is rewritten by the next batch
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c) {
+      const int64_t r = first + c * 64 + lane;
+      const uint64_t mask = __ballot(v[c] != 0);    // zero for chunks past the end
+      if (c < n_chunks && r < a.n) {
+        if (v[c] != 0) {
+          a.row_index[pos + __builtin_popcountll(mask & below)] = (int32_t)r;
+        } else {
+          for (int o = 0; o < n_outs; ++o) outs[o][r] = 0.f;
+          if (a.out_argmax) a.out_argmax[r] = -1;
+        }
+      }
+      pos += __builtin_popcountll(mask);
+    }
+    done += total;
   }
-  if (tid == 1023) *a.n_valid = base + inc;
-  if (wave == 15) {  // the last wave knows the total: it also fixes the work decomposition
-    const int total = __shfl(base + inc, 63, 64);
-    const FusedSchedule sch = fused_schedule_wave(total, a.bt, a.slots, a.n_vtiles, lane);
+  if (tid == 0) *a.n_valid = done;
+  if (wave == 15) {  // one wave also fixes the work decomposition, which depends on the total
+    const FusedSchedule sch = fused_schedule_wave(done, a.bt, a.slots, a.n_vtiles, lane);
     if (lane == 0) *reinterpret_cast<FusedSchedule*>(a.n_valid + 4) = sch;
   }
 }
