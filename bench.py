@@ -339,7 +339,7 @@ def bench_dual(dev, steps, warmup, n=32 * 2048, H=4096):
     return tm
 
 
-def bench_ceiling(dev, steps, warmup, operands="random"):
+def bench_ceiling(dev, steps, warmup, operands="random", with_requests=False):
     """The fused kernel's LDS -> MFMA inner loop alone (tome_probe_mfma_ceiling): one workgroup per CU, operands
     copied into LDS once, no global loads, barriers or epilogue in the loop.  `random`: W rows ~N(0, 0.02^2) and
     token rows ~N(0, 1) as in config 3; `constant`: every operand 1.0."""
@@ -359,7 +359,7 @@ def bench_ceiling(dev, steps, warmup, operands="random"):
     stream = torch.cuda.current_stream(dev).cuda_stream
 
     def step():
-        _lib.check(lib.tome_probe_mfma_ceiling(ops.data_ptr(), n_wg, k_steps, sink.data_ptr(), stream))
+        _lib.check(lib.tome_probe_mfma_ceiling(ops.data_ptr(), n_wg, k_steps, 1 if with_requests else 0, sink.data_ptr(), stream))
     step()
     torch.cuda.synchronize()
     assert torch.isfinite(sink).all()
@@ -589,13 +589,15 @@ def main():
     if "ceiling" in only:
         t = bench_ceiling(dev, K, W, "random")
         c = bench_ceiling(dev, K, W, "constant")
+        q = bench_ceiling(dev, K, W, "random", with_requests=True)
         SUSTAINED["tflops"] = t["flop"] / (t["ms"] * 1e-3) / 1e12
         legs["mfma_ceiling"] = {
             "value": SUSTAINED["tflops"], "unit": "TFLOP/s", **timing_fields(t), "dtype": "bf16 x bf16 -> f32",
             "config": {"workload": "bare LDS -> MFMA loop of the fused kernel (256x256 workgroup tile, v_mfma_f32_16x16x32_bf16, "
                                    "one workgroup per CU, operands resident in LDS): random operands as in config 3",
                        "workgroups": t["workgroups"], "k_slabs_per_launch": t["k_steps"],
-                       "constant_operands_tflops": c["flop"] / (c["ms"] * 1e-3) / 1e12},
+                       "constant_operands_tflops": c["flop"] / (c["ms"] * 1e-3) / 1e12,
+                       "random_operands_with_fill_requests_tflops": q["flop"] / (q["ms"] * 1e-3) / 1e12},
             "roofline": {"bound": "mfma", "achieved": SUSTAINED["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": SUSTAINED["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "kernel": "mfma_ceiling_kernel",
                          "flop_per_launch": t["flop"]}}

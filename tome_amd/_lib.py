@@ -47,7 +47,7 @@ SIGNATURES = {
     "tome_grpo_pair": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                c_int64, c_int64, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_size_t, c_void_p]),
-    "tome_probe_mfma_ceiling": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
+    "tome_probe_mfma_ceiling": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "tome_lora_merge_workspace": (c_size_t, [c_void_p, c_int64]),
     "tome_lora_merge": (c_int, [c_void_p, c_int64, c_void_p, c_size_t, c_void_p]),
 }

@@ -6,6 +6,10 @@
 // the part puts on any bf16 GEMM of this tiling; with constant operands the same loop runs near the
 // published peak, which shows that the loop itself is not what holds the random case back.
 //
+// With `with_requests` every wave also issues the fused kernel's eight global -> LDS requests per K slab (1 KB each,
+// re-reading the 64 KB operand buffer, which stays in the caches; the data lands in a second LDS region that is never
+// read): what the fill costs by being issued and returned at all, apart from what the L2 side adds in the real kernel.
+//
 // No counterpart in the reference (it has no matrix-core code); bench.py reports the figure next to the
 // published peak as `sustained_peak`.
 #include "common.hpp"
@@ -27,6 +31,16 @@ __device__ __forceinline__ void probe_pair_reads() {
   }
 }
 
+template <int N>
+__device__ __forceinline__ void probe_pair_dma() {
+#pragma unroll
+  for (int q = 0; q < N; ++q) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM (DMA request)
+  }
+}
+
+template <bool REQ>
 __global__ __launch_bounds__(kProbeWG) void mfma_ceiling_kernel(const u32x4* operands, int steps, float* sink) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -64,27 +78,62 @@ __global__ __launch_bounds__(kProbeWG) void mfma_ceiling_kernel(const u32x4* ope
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i0 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], acc[i0 + i][j], 0, 0, 0);
   };
+  // Requests (REQ): piece p of a wave fetches 1 KB of the operand buffer into the second 64 KB of LDS, 4 + 2 + 2 per
+  // step in the quarters where the fused kernel issues them, at most one slab's worth in flight.
+  const char* req_src = reinterpret_cast<const char*>(operands) + wave * 8192 + lane * 16;
+  char* req_dst = smem + kProbeSlabBytes + wave * 1024;
+  auto request = [&](int piece) {
+    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(req_src + piece * 1024),
+                                     (__attribute__((address_space(3))) uint32_t*)(req_dst + piece * 8192), 16, 0, 0);
+  };
   for (int s = 0; s < steps; ++s) {  // one step = one 64-wide K slab = 64 MFMAs per wave
     __builtin_amdgcn_sched_barrier(0);
     read_a(0, 4, fa_hi);
+    if constexpr (REQ) {
+      request(4);
+      request(5);
+    }
     mfma_half(0, fa_lo, fb0);
     probe_pair_reads<2, 4>();
+    if constexpr (REQ) probe_pair_dma<2>();
     __builtin_amdgcn_sched_barrier(0);
     read_a(1, 0, fa_lo);
     read_b(1, fb1);
+    if constexpr (REQ) {
+      request(6);
+      request(7);
+    }
     mfma_half(4, fa_hi, fb0);
-    probe_pair_reads<2, 8>();
+    if constexpr (REQ) {
+      probe_pair_reads<1, 8>();
+      probe_pair_dma<2>();
+    } else {
+      probe_pair_reads<2, 8>();
+    }
     __builtin_amdgcn_sched_barrier(0);
     read_a(1, 4, fa_hi);
     mfma_half(0, fa_lo, fb1);
     probe_pair_reads<2, 4>();
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (REQ) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the fused kernel's wait before its barrier
     read_a(0, 0, fa_lo);
     read_b(0, fb0);
+    if constexpr (REQ) {
+      request(0);
+      request(1);
+      request(2);
+      request(3);
+    }
     mfma_half(4, fa_hi, fb1);
-    probe_pair_reads<2, 8>();
+    if constexpr (REQ) {
+      probe_pair_reads<1, 8>();
+      probe_pair_dma<4>();
+    } else {
+      probe_pair_reads<2, 8>();
+    }
     __builtin_amdgcn_sched_barrier(0);
   }
+  if constexpr (REQ) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no request may outlive the workgroup's LDS
   float total = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i)
@@ -95,15 +144,22 @@ __global__ __launch_bounds__(kProbeWG) void mfma_ceiling_kernel(const u32x4* ope
 
 // `operands`: 64 KB of bf16 (device), `sink`: n_workgroups * 512 floats (device).  FLOP of one launch:
 // n_workgroups * steps * 2 * 256 * 256 * 64.
-hipError_t mfma_probe_launch(const void* operands, int n_workgroups, int steps, float* sink, hipStream_t stream) {
-  static bool attr_set = false;  // opt in to 64 KB of dynamic LDS once
+hipError_t mfma_probe_launch(const void* operands, int n_workgroups, int steps, int with_requests, float* sink,
+                             hipStream_t stream) {
+  static bool attr_set = false;  // opt in to the large dynamic LDS once
   if (!attr_set) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&mfma_ceiling_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              kProbeSlabBytes);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&mfma_ceiling_kernel<false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kProbeSlabBytes);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&mfma_ceiling_kernel<true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kProbeSlabBytes);
     attr_set = true;
   }
-  hipLaunchKernelGGL(mfma_ceiling_kernel, dim3((unsigned)n_workgroups), dim3(kProbeWG), kProbeSlabBytes, stream,
-                     static_cast<const u32x4*>(operands), steps, sink);
+  if (with_requests)
+    hipLaunchKernelGGL(mfma_ceiling_kernel<true>, dim3((unsigned)n_workgroups), dim3(kProbeWG), 2 * kProbeSlabBytes, stream,
+                       static_cast<const u32x4*>(operands), steps, sink);
+  else
+    hipLaunchKernelGGL(mfma_ceiling_kernel<false>, dim3((unsigned)n_workgroups), dim3(kProbeWG), kProbeSlabBytes, stream,
+                       static_cast<const u32x4*>(operands), steps, sink);
   return hipGetLastError();
 }
 
