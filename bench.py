@@ -16,6 +16,12 @@ busy for SETTLE_MS, so that clocks have left their idle state; the count is repo
 `settle_launches`), then times EXACTLY K back-to-back steps between two HIP events on the launch
 stream (`ms_per_step`, the mean), and finally repeats K steps with an event between launches for the
 median of the per-launch times (`median_ms`, `min_ms`; this second pass does not feed `ms_per_step`).
+The matrix-core legs add a clock pass: the same step is queued for CLOCK_MS of GPU time (untimed) and the
+host meanwhile reads the engine clock the driver reports (`pp_dpm_sclk` of the device in sysfs, a
+smoothed value) every few milliseconds; the median of the samples from the second half of that pass
+is `sclk_mhz`, and these legs price themselves against the published peak scaled to that clock as well
+(`roofline.peak_at_sclk`, `roofline.frac_at_sclk`): the published 2.5 PFLOP/s is 256 CUs x 4096 FLOP per clock at the 2.4 GHz peak engine clock, which the part does not
+hold under a matrix-core load on random operands.
 
 Prints ONE JSON line on stdout.  Everything else goes to stderr.
 """
@@ -34,8 +40,10 @@ if ROOT not in sys.path:
 V = 151936
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+PEAK_ENGINE_CLOCK_MHZ = 2400.0  # the clock the published matrix-core figures are quoted at
 SETTLE_MS = 60.0                # untimed GPU-busy time in front of every timed region (default of --settle-ms)
 SETTLE = {"ms": SETTLE_MS}
+CLOCK = {"ms": 400.0}           # GPU-busy time of the clock pass of the matrix-core legs (--clock-ms; 0 = none)
 SETTLE_MAX_LAUNCHES = 2000
 LEGS = ["row", "config1", "ceiling", "fused", "gemm", "config4", "config5", "small", "midsize", "decode", "lora"]
 SUSTAINED = {"tflops": None}    # bf16 MFMA rate of the probe loop on random operands, measured by the `ceiling` leg
@@ -83,7 +91,43 @@ def make_config2(dev, seed=1234):
     return logits, targets, lengths, spike
 
 
-def time_steps(fn, steps, warmup):
+_SCLK = {"path": False}
+
+
+def sclk_path():
+    """sysfs file with the engine clock levels of the GPU that torch calls device 0, or None."""
+    if _SCLK["path"] is False:
+        import glob
+        import torch
+        found = None
+        try:
+            pr = torch.cuda.get_device_properties(0)
+            want = "%04x:%02x:%02x." % (pr.pci_domain_id, pr.pci_bus_id, pr.pci_device_id)
+            paths = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+            hits = [q for q in paths if want in os.path.realpath(os.path.dirname(q))]
+            found = hits[0] if hits else (paths[0] if len(paths) == 1 else None)
+        except Exception:  # noqa: BLE001 - the clock is an optional extra
+            found = None
+        _SCLK["path"] = found
+    return _SCLK["path"]
+
+
+def read_sclk_mhz():
+    """The level the driver marks as current ('1: 1836Mhz *'), in MHz, or None."""
+    path = sclk_path()
+    if not path:
+        return None
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.rstrip().endswith("*"):
+                    return float(line.split(":")[1].strip().split("Mhz")[0])
+    except (OSError, ValueError, IndexError):
+        return None
+    return None
+
+
+def time_steps(fn, steps, warmup, clock=False):
     """Warm-up, settle, timed region, per-launch pass (see the module docstring).  Times in milliseconds by
     HIP events recorded on the stream the kernels run on (torch's current stream, which the library
     launches into)."""
@@ -122,13 +166,32 @@ def time_steps(fn, steps, warmup):
         ev[i + 1].record()
     torch.cuda.synchronize()
     per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(steps))
+    clocks = []   # clock pass: the engine clock while the same step keeps the GPU busy for CLOCK["ms"]
+    if clock and CLOCK["ms"] > 0 and sclk_path():
+        n = max(steps, int(CLOCK["ms"] / mean_ms) + 1)
+        done = torch.cuda.Event()
+        t1 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        done.record()
+        while not done.query():
+            c = read_sclk_mhz()
+            if c and not done.query():
+                clocks.append((time.perf_counter() - t1, c))
+            time.sleep(0.003)
+        torch.cuda.synchronize()
+        half = (time.perf_counter() - t1) / 2
+        clocks = sorted(c for (at, c) in clocks if at >= half)
     return {"ms": mean_ms, "wall_ms": wall_ms, "median_ms": per[len(per) // 2], "min_ms": per[0],
-            "settle_launches": settle}
+            "settle_launches": settle, "sclk_mhz": clocks[len(clocks) // 2] if clocks else None}
 
 
 def timing_fields(t):
-    return {"ms_per_step": t["ms"], "median_ms": t["median_ms"], "min_ms": t["min_ms"],
-            "settle_launches": t["settle_launches"]}
+    d = {"ms_per_step": t["ms"], "median_ms": t["median_ms"], "min_ms": t["min_ms"],
+         "settle_launches": t["settle_launches"]}
+    if t.get("sclk_mhz"):
+        d["sclk_mhz"] = t["sclk_mhz"]
+    return d
 
 
 def hbm_roofline(nbytes, ms, traffic, kernel):
@@ -137,10 +200,13 @@ def hbm_roofline(nbytes, ms, traffic, kernel):
             "traffic": traffic, "kernel": kernel, "bytes_per_launch": nbytes}
 
 
-def mfma_roofline(flop, ms, traffic, kernel):
+def mfma_roofline(flop, ms, traffic, kernel, sclk_mhz=None):
     tf = flop / (ms * 1e-3) / 1e12
     r = {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
          "frac": tf / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic, "kernel": kernel, "flop_per_launch": flop}
+    if sclk_mhz:   # the published peak at the engine clock the part held during this leg
+        r["peak_at_sclk"] = MFMA_BF16_PEAK_TFLOPS * sclk_mhz / PEAK_ENGINE_CLOCK_MHZ
+        r["frac_at_sclk"] = tf / r["peak_at_sclk"]
     if SUSTAINED["tflops"]:   # what the bare LDS -> MFMA loop reaches on random bf16 operands, same run (`ceiling` leg)
         r["sustained_peak"] = SUSTAINED["tflops"]
         r["frac_of_sustained"] = tf / SUSTAINED["tflops"]
@@ -273,7 +339,7 @@ def bench_fused(dev, steps, warmup, n=4096, H=1024, temperature=1.0, lengths=Non
     ref = ref[torch.arange(idx.numel(), device=dev), targets[idx].long()]
     assert (lp[idx] - ref).abs().max().item() < 2e-3
     del ref
-    tm = time_steps(step, steps, warmup)
+    tm = time_steps(step, steps, warmup, clock=True)
     tm.update({"tokens": n, "valid": n_valid, "H": H, "flop": 2.0 * n_valid * H * V,
                "bytes": V * H * 2 + n_valid * H * 2})
     return tm
@@ -293,7 +359,7 @@ def bench_library_gemm(dev, steps, warmup, n=4096, H=1024):
         torch.mm(hidden, wt, out=out)
     step()
     torch.cuda.synchronize()
-    tm = time_steps(step, steps, warmup)
+    tm = time_steps(step, steps, warmup, clock=True)
     tm.update({"tokens": n, "H": H, "flop": 2.0 * n * H * V})
     return tm
 
@@ -334,7 +400,7 @@ def bench_dual(dev, steps, warmup, n=32 * 2048, H=4096):
     for w, got in ((w_pol, lp), (w_ref, ref_lp)):       # gate: 32 rows of each weight set against fp32 torch
         ref = torch.log_softmax(hidden[idx].float() @ w.float().T, dim=-1)[torch.arange(32, device=dev), targets[idx].long()]
         assert (got[idx] - ref).abs().max().item() < 2e-3
-    tm = time_steps(step, steps, warmup)
+    tm = time_steps(step, steps, warmup, clock=True)
     tm.update({"tokens": n, "H": H, "flop": 2.0 * 2.0 * n * H * V, "bytes": 2 * V * H * 2 + n * H * 2})
     return tm
 
@@ -363,7 +429,7 @@ def bench_ceiling(dev, steps, warmup, operands="random", with_requests=False):
     step()
     torch.cuda.synchronize()
     assert torch.isfinite(sink).all()
-    tm = time_steps(step, steps, warmup)
+    tm = time_steps(step, steps, warmup, clock=True)
     tm.update({"flop": float(n_wg) * k_steps * 2 * 256 * 256 * 64, "workgroups": n_wg, "k_steps": k_steps})
     return tm
 
@@ -498,6 +564,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
                     help="untimed GPU-busy time in front of every timed region (counter runs pass 0)")
+    ap.add_argument("--clock-ms", type=float, default=CLOCK["ms"],
+                    help="GPU-busy time of the clock pass after each matrix-core leg (0 = none; profiling runs pass 0)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None, help="comma-separated subset of: " + ", ".join(LEGS))
     ap.add_argument("--row-variant", choices=["both", "mask", "list", "all"], default="both",
@@ -535,6 +603,7 @@ def main():
         del src, dst
     K, W = args.steps, args.warmup
     SETTLE["ms"] = args.settle_ms
+    CLOCK["ms"] = args.clock_ms
     legs = {}   # name -> JSON object; the first one present also becomes the top-level line
 
     def done(name):
@@ -597,10 +666,12 @@ def main():
                                    "one workgroup per CU, operands resident in LDS): random operands as in config 3",
                        "workgroups": t["workgroups"], "k_slabs_per_launch": t["k_steps"],
                        "constant_operands_tflops": c["flop"] / (c["ms"] * 1e-3) / 1e12,
-                       "random_operands_with_fill_requests_tflops": q["flop"] / (q["ms"] * 1e-3) / 1e12},
-            "roofline": {"bound": "mfma", "achieved": SUSTAINED["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": SUSTAINED["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "kernel": "mfma_ceiling_kernel",
-                         "flop_per_launch": t["flop"]}}
+                       "constant_operands_sclk_mhz": c.get("sclk_mhz"),
+                       "random_operands_with_fill_requests_tflops": q["flop"] / (q["ms"] * 1e-3) / 1e12,
+                       "random_operands_with_fill_requests_sclk_mhz": q.get("sclk_mhz")},
+            "roofline": mfma_roofline(t["flop"], t["ms"], None, "mfma_ceiling_kernel", t.get("sclk_mhz"))}
+        legs["mfma_ceiling"]["roofline"].pop("sustained_peak", None)
+        legs["mfma_ceiling"]["roofline"].pop("frac_of_sustained", None)
         done("mfma_ceiling")
     if "fused" in only:
         t = bench_fused(dev, K, W)
@@ -609,7 +680,7 @@ def main():
             "dtype": "bf16 x bf16 -> f32",
             "config": {"workload": "config 3: fused lm_head + log-softmax, hidden [4096,1024] x W [151936,1024] bf16",
                        "tokens": t["tokens"], "hidden": t["H"], "vocab": V, "temperature": 1.0},
-            "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("fused_lmhead_config3"), "fused_lmhead_dma_kernel")}
+            "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("fused_lmhead_config3"), "fused_lmhead_dma_kernel", t.get("sclk_mhz"))}
         done("fused_lmhead")
     if "gemm" in only:
         t = bench_library_gemm(dev, K, W)
@@ -617,7 +688,7 @@ def main():
             "value": t["flop"] / (t["ms"] * 1e-3) / 1e12, "unit": "TFLOP/s", **timing_fields(t), "dtype": "bf16 x bf16 -> bf16",
             "config": {"workload": "for scale, not part of the path: torch.mm (vendor GEMM library) on config 3's shape, bf16 logits "
                                    "[4096, 151936] written, no softmax", "tokens": t["tokens"], "hidden": t["H"], "vocab": V},
-            "roofline": mfma_roofline(t["flop"], t["ms"], None, "vendor library GEMM (hipBLASLt / rocBLAS via torch.mm)")}
+            "roofline": mfma_roofline(t["flop"], t["ms"], None, "vendor library GEMM (hipBLASLt / rocBLAS via torch.mm)", t.get("sclk_mhz"))}
         done("library_gemm_config3")
     if "config4" in only:
         t = bench_fused(dev, K, W, n=16 * 1024, H=2560, temperature=0.7, lengths=(16, 1024, 128, 1024), seed=444)
@@ -627,7 +698,7 @@ def main():
             "config": {"workload": "config 4: fused lm_head + log-softmax, hidden [16x1024, 2560] x W [151936, 2560] bf16, "
                                    "temperature 0.7, sequence lengths~U[128,1024] as a padding mask (FLOP counted on valid tokens)",
                        "tokens": t["tokens"], "valid_tokens": t["valid"], "hidden": t["H"], "vocab": V, "temperature": 0.7},
-            "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("fused_lmhead_config4"), "fused_lmhead_dma_kernel")}
+            "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("fused_lmhead_config4"), "fused_lmhead_dma_kernel", t.get("sclk_mhz"))}
         done("config4_fused_varlen")
     if "config5" in only:
         t = bench_dual(dev, max(3, K // 4), max(1, W // 4))     # 0.1 s per step: a quarter of the steps
@@ -638,7 +709,7 @@ def main():
                                    "(ref = policy + N(0, 0.002^2)); outputs lp, ref_lp, k3, entropy",
                        "tokens": t["tokens"], "hidden": t["H"], "vocab": V, "temperature": 1.0},
             "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("grpo_dual_config5"),
-                                      "fused_lmhead_dma_kernel (two sweeps) + fused_combine_kernel")}
+                                      "fused_lmhead_dma_kernel (two sweeps) + fused_combine_kernel", t.get("sclk_mhz"))}
         done("config5_grpo_dual")
     if "small" in only:
         t = bench_fused(dev, K, W, n=64)
