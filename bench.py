@@ -519,7 +519,7 @@ def cpu_baseline(budget_s=10.0):
     x = (rng.standard_normal((rows, V)) * 2.0).astype(np.float32)
     t = rng.integers(0, V, size=rows).astype(np.int32)
 
-    def median_time(fn, budget, cap=200):
+    def median_time(fn, budget, cap=5000):
         fn()
         times = []
         t_end = time.perf_counter() + budget
