@@ -160,7 +160,8 @@ int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows
  * and the selector below.
  */
 /* Testing and tuning hook, no counterpart in the reference: kind 0 / 1 makes the fused entry points take
- * the generic / LDS-DMA sweep kernel wherever its shape rules allow, -1 (the default) picks by shape.
+ * the generic / LDS-DMA sweep kernel wherever its shape rules allow, 3 / 4 the LDS-DMA kernel with
+ * 256-row / 224-row vocab tiles, -1 (the default, also for any other value) picks by shape.
  * Process-wide; set it while no call of this library is running. */
 void tome_select_fused_kernel(int kind);
 size_t tome_fused_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V);

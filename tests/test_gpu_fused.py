@@ -17,9 +17,10 @@ TOL = 2e-3
 
 @pytest.fixture
 def force_kernel():
-    """tome_select_fused_kernel for one test: 'generic' / 'dma' force that sweep kernel, reset afterwards."""
+    """tome_select_fused_kernel for one test: 'generic' / 'dma' force that sweep kernel, 'dma256' / 'dma224' the
+    LDS-DMA kernel with that vocab-tile height; reset afterwards."""
     lib = tome_amd.load_library()
-    yield lambda kind: lib.tome_select_fused_kernel({"generic": 0, "dma": 1}[kind])
+    yield lambda kind: lib.tome_select_fused_kernel({"generic": 0, "dma": 1, "dma256": 3, "dma224": 4}[kind])
     lib.tome_select_fused_kernel(-1)
 
 
@@ -182,7 +183,7 @@ def test_fused_argmax_spike_and_ties(dev):
     assert (masked.argmax.cpu().numpy() == -1).all()
 
 
-@pytest.mark.parametrize("kind", ["generic", "dma"])
+@pytest.mark.parametrize("kind", ["generic", "dma", "dma256", "dma224"])
 def test_fused_every_kernel_path(dev, kind, force_kernel):
     """The two GEMM kernels behind tome_fused_lmhead_logprob (generic / LDS-DMA) are picked
     by shape; tome_select_fused_kernel forces each of them onto the same problem."""
@@ -201,7 +202,32 @@ def test_fused_every_kernel_path(dev, kind, force_kernel):
     assert (r.lp.cpu().numpy()[~m] == 0).all() and (r.argmax.cpu().numpy()[~m] == -1).all()
 
 
-@pytest.mark.parametrize("kind", ["generic", "dma"])
+@pytest.mark.parametrize("n,H,V", [(50, 128, 224 * 3), (100, 192, 224 * 5 + 7), (256, 1024, 20000), (200, 64, 223), (1000, 256, 4481)])
+def test_fused_tile_heights_agree(dev, n, H, V, force_kernel):
+    """The LDS-DMA kernel with 256-row and with 224-row vocab tiles (64-, 128- and 256-token tiles): each against the
+    oracle, targets placed on the first and last rows of 224-row and 256-row tiles, and the argmax of both equal."""
+    h, w, t = _inputs(dev, n, H, V, seed=n + V, w_scale=0.1)
+    edges = [v for v in (0, 111, 112, 223, 224, 255, 256, 447, 448, V - 1) if v < V]
+    t[: len(edges)] = edges
+    valid = np.ones(n, dtype=np.int32)
+    valid[n // 3] = 0
+    want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(w), t, 0.9)
+    got = {}
+    for kind in ("dma256", "dma224"):
+        force_kernel(kind)
+        r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 0.9, want_lse=True, want_entropy=True,
+                                           want_argmax=True, row_valid=torch.from_numpy(valid).to(dev))
+        m = valid.astype(bool)
+        np.testing.assert_allclose(r.lp.cpu().numpy()[m], want["lp"][m], atol=TOL, rtol=0)
+        np.testing.assert_allclose(r.lse.cpu().numpy()[m], want["lse"][m], atol=TOL, rtol=0)
+        np.testing.assert_allclose(r.entropy.cpu().numpy()[m], want["entropy"][m], atol=TOL, rtol=0)
+        check_argmax(h, w, r.argmax.cpu().numpy(), want, 0.9, rows=np.flatnonzero(m), min_clear=0.0)
+        assert r.lp.cpu().numpy()[n // 3] == 0 and r.argmax.cpu().numpy()[n // 3] == -1
+        got[kind] = r.argmax.cpu().numpy()
+    np.testing.assert_array_equal(got["dma256"], got["dma224"])
+
+
+@pytest.mark.parametrize("kind", ["generic", "dma", "dma224"])
 @pytest.mark.parametrize("n,frac_valid", [(300, 1.0), (2304, 1.0), (9000, 1.0), (9000, 0.45), (20000, 0.8)])
 def test_fused_every_partial_is_written(dev, kind, n, frac_valid, force_kernel):
     """The work decomposition (token tiles x vocab splits, one or several rounds of workgroups, chosen on

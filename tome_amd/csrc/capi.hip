@@ -218,7 +218,9 @@ static int check_fused(const void* hidden, const void* w, int64_t n_tokens, int6
   return TOME_OK;
 }
 
-void tome_select_fused_kernel(int kind) { tome::fused_force_kernel(kind < 0 || kind > 1 ? -1 : kind); }
+void tome_select_fused_kernel(int kind) {
+  tome::fused_force_kernel(kind == 0 || kind == 1 || kind == 3 || kind == 4 ? kind : -1);
+}
 
 size_t tome_fused_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V) {
   if (n_tokens <= 0 || H <= 0 || V <= 0) return 0;

@@ -571,9 +571,17 @@ __device__ __forceinline__ void pair_reads() {
   }
 }
 
-template <bool ENT, bool AMAX, int NBT>
+// HI: vocab blocks in the second half of a wave's tile, 4 or 3.  With 3 the workgroup tile is 224 vocab rows (2 x 7 blocks)
+// instead of 256: the schedule takes it where whole 256-row tiles would leave the workgroups of a launch that streams W
+// once with uneven shares (594 tiles over 256 workgroups: three for some, two for the others).  The slab keeps its 256
+// rows in LDS; the 32 unused ones are requested as copies of rows the same instruction fetches anyway.
+template <bool ENT, bool AMAX, int NBT, int HI>
 __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
+  static_assert(HI == 4 || HI == 3, "tile heights: 256 or 224 vocab rows");
+  constexpr int kNBVw = 4 + HI;                     // 16-row vocab blocks per wave
+  constexpr int kWaveRows = kNBVw * 16;             // vocab rows per wave
+  constexpr int kTileRows = 2 * kWaveRows;          // vocab rows per workgroup tile
   constexpr int k2NBT = NBT;                        // 16-token blocks per wave
   constexpr int k2BT = dma_tile_tokens(NBT);        // tokens per workgroup
   constexpr int kWaveTok = NBT * 16;                // tokens per wave
@@ -617,7 +625,11 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   auto point_a = [&](int vt) {  // rows past V (last tile only) read the last row; masked in the epilogue
 #pragma unroll
     for (int j = 0; j < k2Loads; ++j) {
-      int64_t v = (int64_t)vt * k2BV + (j * 8 + wave) * 8 + dr;
+      int64_t v = (int64_t)vt * kTileRows + (j * 8 + wave) * 8 + dr;  // tile row = LDS row of the slab
+      if constexpr (HI != 4) {  // LDS rows past the tile: a copy of what waves 0-3 request with this instruction
+        const int r = (j * 8 + wave) * 8 + dr;
+        v = (int64_t)vt * kTileRows + (r < kTileRows ? r : r - 32);
+      }
       v = v < a.V ? v : a.V - 1;
       pa[j] = a.weight + v * a.weight_stride_b + dc * 16;
     }
@@ -647,7 +659,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 
   // ---- fragment read offsets inside a slab (swizzled): lane group g reads chunk 4*ks + g ----------
   const int swz = (g ^ ((l16 >> 1) & 7)) * 16;  // sub-step k0; k1 is this ^ 64
-  const int rdA = (wave_v * kWaveV + l16) * k2RowBytes + swz;
+  const int rdA = (wave_v * kWaveRows + l16) * k2RowBytes + swz;  // kWaveRows is a multiple of 16: the swizzle term stays l16's
   const int rdB = (wave_t * kWaveTok + l16) * k2RowBytes + swz;
 
   const int nk = a.H / k2BK;
@@ -680,13 +692,15 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
       if (i_vt < vt1) point_a(i_vt);
     }
   };
-  // Fragments of one K = 32 sub-step of a slab: W blocks [i0, i0 + 4) or the hidden blocks.
-  auto read_a = [&](int slot, int ks, int i0, bf16x8 (&fa)[4]) {
+  // Fragments of one K = 32 sub-step of a slab: W blocks [i0, i0 + n) or the hidden blocks.
+  auto read_a = [&](int slot, int ks, int i0, bf16x8 (&fa)[4], auto n) {
     const char* slab = smem + ((unsigned)slot % kBufs) * kWBytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < decltype(n)::value; ++i)
       fa[i] = *reinterpret_cast<const bf16x8*>(slab + (rdA ^ (ks * 64)) + (i0 + i) * 16 * k2RowBytes);
   };
+  constexpr std::integral_constant<int, 4> kLo{};
+  constexpr std::integral_constant<int, HI> kHi{};
   auto read_b = [&](int slot, int ks, bf16x8 (&fb)[k2NBT]) {
     const char* slab = smem + kHBase + ((unsigned)slot % kBufs) * kHBytes;
 #pragma unroll
@@ -709,25 +723,25 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   __builtin_amdgcn_s_barrier();
 
   bf16x8 fa_lo[4], fa_hi[4], fb0[k2NBT], fb1[k2NBT];
-  read_a(0, 0, 0, fa_lo);
+  read_a(0, 0, 0, fa_lo, kLo);
   read_b(0, 0, fb0);
 
-  f32x4v acc[k2NBV][k2NBT];
+  f32x4v acc[kNBVw][k2NBT];
 #pragma unroll
-  for (int i = 0; i < k2NBV; ++i)
+  for (int i = 0; i < kNBVw; ++i)
 #pragma unroll
     for (int j = 0; j < k2NBT; ++j)
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
-  // 16 MFMAs on four vocab blocks; the group barriers then put one LDS read or DMA request behind
+  // 16 (12) MFMAs on four (three) vocab blocks; the group barriers then put one LDS read or DMA request behind
   // every MFMA (or every second one), so that its issue hides under the MFMA's execution.
   // `fresh`: the first K sub-step of a vocab tile starts from a zero C operand, which saves clearing
   // the 128 accumulator registers after every fold.
-  auto mfma_half = [&](int i0, bf16x8 (&fa)[4], bf16x8 (&fb)[k2NBT], auto fresh) {
+  auto mfma_half = [&](int i0, bf16x8 (&fa)[4], bf16x8 (&fb)[k2NBT], auto fresh, auto n) {
     const f32x4v zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < decltype(n)::value; ++i)
 #pragma unroll
       for (int j = 0; j < k2NBT; ++j)
         acc[i0 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], decltype(fresh)::value ? zero : acc[i0 + i][j],
@@ -744,22 +758,22 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   };
   auto do_step = [&](auto fresh) {
     __builtin_amdgcn_sched_barrier(0);
-    read_a(step, 0, 4, fa_hi);
+    read_a(step, 0, 4, fa_hi, kHi);
 #pragma unroll
     for (int piece = kP4; piece < kP4 + kP1; ++piece) issue_piece(piece);  // second portion of the request for slab step + 1
-    mfma_half(0, fa_lo, fb0, fresh);
+    mfma_half(0, fa_lo, fb0, fresh, kLo);
     if constexpr (NBT == 4) {
-      pair_reads<2, 4>();
+      pair_reads<2, HI>();
       pair_dma(std::integral_constant<int, kP1>{});
     }
     __builtin_amdgcn_sched_barrier(0);
-    read_a(step, 1, 0, fa_lo);
+    read_a(step, 1, 0, fa_lo, kLo);
     read_b(step, 1, fb1);
 #pragma unroll
     for (int piece = kP4 + kP1; piece < k2DmaPerSlab; ++piece) issue_piece(piece);  // third portion
-    mfma_half(4, fa_hi, fb0, fresh);
+    mfma_half(4, fa_hi, fb0, fresh, kHi);
     if constexpr (NBT == 4) {
-      if constexpr (kP2 == 0) {
+      if constexpr (kP2 == 0 && HI == 4) {
         pair_reads<2, 8>();
       } else {
         pair_reads<1, 8>();
@@ -768,9 +782,9 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (kP4 < k2DmaPerSlab) issue_done();
-    read_a(step, 1, 4, fa_hi);
-    mfma_half(0, fa_lo, fb1, std::false_type{});
-    if constexpr (NBT == 4) pair_reads<2, 4>();
+    read_a(step, 1, 4, fa_hi, kHi);
+    mfma_half(0, fa_lo, fb1, std::false_type{}, kLo);
+    if constexpr (NBT == 4) pair_reads<2, HI>();
     __builtin_amdgcn_sched_barrier(0);
     // This wave has read all it needs of slab `step` and its share of slab step+1 has landed; after
     // the (fence-less) barrier both hold for everyone.  (With three buffers the request of slab step+2
@@ -781,11 +795,11 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     // first portion of the next request, which refills the buffers of slab `step`.  The DMA requests write
     // LDS, so they keep their program order after the fragment reads.
     __builtin_amdgcn_sched_barrier(0);
-    read_a(step + 1, 0, 0, fa_lo);
+    read_a(step + 1, 0, 0, fa_lo, kLo);
     read_b(step + 1, 0, fb0);
 #pragma unroll
     for (int piece = 0; piece < kP4; ++piece) issue_piece(piece);
-    mfma_half(4, fa_hi, fb1, std::false_type{});
+    mfma_half(4, fa_hi, fb1, std::false_type{}, kHi);
     if constexpr (NBT == 4) {
       pair_reads<1, 8>();
       pair_dma(std::integral_constant<int, kP4>{});
@@ -798,8 +812,8 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   for (int vt = vt0; vt < vt1; ++vt) {
     do_step(std::true_type{});
     for (int kt = 1; kt < nk; ++kt) do_step(std::false_type{});
-    const int v0 = vt * k2BV;
-    fold_tile16<ENT, AMAX>(acc, st, tx, tgt, v0 + wave_v * kWaveV, g, v0 + k2BV > a.V, a.V, a.scale);
+    const int v0 = vt * kTileRows;
+    fold_tile16<ENT, AMAX>(acc, st, tx, tgt, v0 + wave_v * kWaveRows, g, v0 + kTileRows > a.V, a.V, a.scale);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no request may outlive the workgroup's LDS
 
@@ -1150,6 +1164,7 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
 // with the batch.  Decode-sized batches whose hidden states fit the waves' registers take the streaming kernel.
 
 enum FusedKind { kGeneric = 0, kDma = 1, kSmall = 2 };
+constexpr int kForceDma256 = 3, kForceDma224 = 4;  // selector values: the DMA kernel with one tile height
 
 // Kernel selector for tests and tuning runs: -1 (the default) picks by shape, kGeneric / kDma force that
 // sweep kernel wherever its shape rules allow.  Process-wide; set it while no call is in flight.
@@ -1159,6 +1174,7 @@ void fused_force_kernel(int kind) { g_forced_kind.store(kind, std::memory_order_
 struct FusedPlan {
   FusedKind kind;
   int dma_nbt;                               // kDma only: token blocks per wave (4, 2 or 1: 256, 128 or 64 tokens per tile)
+  int dma_hi;                                // kDma only: 4 = 256-row vocab tiles, 3 = 224-row ones
   int small_nbt, small_ksteps, small_waves;  // kSmall only
   int bt, bv, slots, n_vtiles;
   int grid;            // workgroups to launch: the most any number of valid tokens can ask for
@@ -1219,9 +1235,10 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   if (H % k2BK == 0) p.kind = kDma;
   // The streaming kernel runs one workgroup per CU: without a CU count (no device) the tiled kernels serve.
   if (small_shape(n_tokens, H, V, p.small_nbt, p.small_ksteps, p.small_waves) && small_wg_count() >= 2) p.kind = kSmall;
+  p.dma_hi = 4;
   const int forced = g_forced_kind.load(std::memory_order_relaxed);
   if (forced == kGeneric) p.kind = kGeneric;
-  if (forced == kDma && H % k2BK == 0) p.kind = kDma;
+  if ((forced == kDma || forced == kForceDma256 || forced == kForceDma224) && H % k2BK == 0) p.kind = kDma;
   p.n_vtiles = 0;
   if (p.kind == kSmall) {
     // One partial per (token, workgroup); one workgroup per CU, at most 512.
@@ -1235,6 +1252,25 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   }
   p.bt = p.kind == kGeneric ? kBT : dma_tile_tokens(p.dma_nbt);   // the DMA path: 256 vocab rows x 256, 128 or 64 tokens
   p.bv = p.kind == kGeneric ? kBV : k2BV;
+  if (p.kind == kDma) {
+    // Tile height.  Where one round of workgroups streams W once, what counts is the longest vocab range in ROWS: whole
+    // 256-row tiles deal V = 151936 as three tiles to 82 workgroups and two to the others, 224-row tiles as three to 167
+    // and two to 89 - an eighth less for the longest.  The shorter tile moves 1/7 more hidden-state bytes per MAC, so it
+    // has to win by more than that is worth (8 %), and it is only considered in the one-round regime.
+    const int tt = fused_ttiles((int)n_tokens, p.bt);
+    if (forced == kForceDma224) {
+      p.dma_hi = 3;
+    } else if (forced != kForceDma256 && tt * 8 <= 256) {
+      const int sp = fused_one_round_splits(tt, 256, 1 << 30);
+      auto longest_rows = [&](int rows) {
+        const int64_t nvt = V > 0 ? (V + rows - 1) / rows : 1;
+        const int64_t s = sp < nvt ? sp : nvt;
+        return ((nvt + s - 1) / s) * rows;
+      };
+      if (longest_rows(224) * 108 < longest_rows(256) * 100) p.dma_hi = 3;
+    }
+    if (p.dma_hi == 3) p.bv = 224;
+  }
   // resident workgroups on 256 CUs: 2 per CU, or 1 for the DMA path (80-128 KB of LDS; two 64-token workgroups of 80 KB
   // per CU measured slower than one: 288 against 277 us at 64 x 4096)
   p.slots = p.kind == kGeneric ? 512 : 256;
@@ -1270,21 +1306,26 @@ size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weigh
   return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, H, V) + normed_bytes(n_tokens, H, with_norm);
 }
 
-template <bool ENT, bool AMAX, int NBT>
+template <bool ENT, bool AMAX, int NBT, int HI>
 static void launch_dma_nbt(const FusedArgs& a, int grid, hipStream_t stream) {
   static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
   if (!attr_set) {
-    allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX, NBT>, dma_lds_bytes(NBT));
+    allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI>, dma_lds_bytes(NBT));
     attr_set = true;
   }
-  hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX, NBT>), dim3((unsigned)grid), dim3(k2WG), dma_lds_bytes(NBT), stream,
-                     a);
+  hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI>), dim3((unsigned)grid), dim3(k2WG), dma_lds_bytes(NBT),
+                     stream, a);
+}
+template <bool ENT, bool AMAX, int HI>
+static void launch_dma_hi(const FusedArgs& a, int nbt, int grid, hipStream_t stream) {
+  if (nbt == 4) launch_dma_nbt<ENT, AMAX, 4, HI>(a, grid, stream);
+  else if (nbt == 2) launch_dma_nbt<ENT, AMAX, 2, HI>(a, grid, stream);
+  else launch_dma_nbt<ENT, AMAX, 1, HI>(a, grid, stream);
 }
 template <bool ENT, bool AMAX>
-static void launch_dma(const FusedArgs& a, int nbt, int grid, hipStream_t stream) {
-  if (nbt == 4) launch_dma_nbt<ENT, AMAX, 4>(a, grid, stream);
-  else if (nbt == 2) launch_dma_nbt<ENT, AMAX, 2>(a, grid, stream);
-  else launch_dma_nbt<ENT, AMAX, 1>(a, grid, stream);
+static void launch_dma(const FusedArgs& a, int nbt, int hi, int grid, hipStream_t stream) {
+  if (hi == 3) launch_dma_hi<ENT, AMAX, 3>(a, nbt, grid, stream);
+  else launch_dma_hi<ENT, AMAX, 4>(a, nbt, grid, stream);
 }
 
 template <bool ENT, bool AMAX, int NBT, int KSTEPS>
@@ -1322,8 +1363,8 @@ static int launch_main(const FusedArgs& a, const FusedPlan& plan, bool want_argm
     return n;  // >= 2: fused_plan only picks this kernel when it can be placed
   }
   if (plan.kind == kDma) {
-    if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.grid, stream);
-    else launch_dma<ENT, false>(a, plan.dma_nbt, plan.grid, stream);
+    if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.dma_hi, plan.grid, stream);
+    else launch_dma<ENT, false>(a, plan.dma_nbt, plan.dma_hi, plan.grid, stream);
   } else {
     if (want_argmax) hipLaunchKernelGGL((fused_lmhead_kernel<ENT, true>), dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
     else hipLaunchKernelGGL((fused_lmhead_kernel<ENT, false>), dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
