@@ -511,9 +511,10 @@ __device__ __forceinline__ void write_partials16(RowStat (&st)[NBT], float (&tx)
 //   * global_load_lds_dwordx4: every lane fetches 16 bytes and the wave's 1 KB lands contiguously
 //     in LDS, bypassing registers.  No staging registers are needed, which leaves room to
 //     double-buffer the MFMA fragments.
-//   * What bounds this kernel is the L2 -> LDS fill (64 KB per 256x256x64 MACs and CU: its requests take
-//     MFMA issue time in proportion to their number, wherever the data lands and whether or not it hits in
-//     L2), and the L2 serves it by the request, not by the byte: a slab row is therefore one whole 128-byte
+//   * What this kernel pays for beside its MFMAs is the L2 -> LDS fill (64 KB per 256x256x64 MACs and CU: the
+//     requests cost in proportion to their number, wherever the data lands and whether or not it hits in L2 -
+//     mostly as engine clock, which this power-limited part lowers under the added load, not as issue slots),
+//     and the L2 serves it by the request, not by the byte: a slab row is therefore one whole 128-byte
 //     cache line (K = 64), which streams 1.5x faster than 64-byte rows.  Two 64 KB slabs (W 256 rows +
 //     hidden 256 rows each) fill the LDS; one is computed on while the other is in flight.  Step s (one
 //     slab = two K = 32 MFMA sub-steps of 32 MFMAs per wave, each in two halves by vocab block) runs
