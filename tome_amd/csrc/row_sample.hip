@@ -507,30 +507,47 @@ __global__ __launch_bounds__(kRowWG) void row_sample_combine_kernel(SampleArgs a
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int k = a.top_k, m = a.splits * k;         // <= 64 * 32 = kSampMergeCap
   const uint64_t* keys = a.part_keys + r * m;      // per split: its k keys in descending order, 0 past the end
-  RowStat st = stat_identity();                    // issued early: overlaps the selection below
+  // Every key is fetched once, up front and together with the statistics: the kernel then waits for global memory
+  // one time (the previous launch wrote these bytes on other dies, so each wait is a trip beyond the L2).
+  constexpr int kPer = kSampMergeCap / kRowWG;
+  uint64_t mine[kPer];
+#pragma unroll
+  for (int q = 0; q < kPer; ++q) {
+    const int i = tid + q * kRowWG;
+    mine[q] = i < m ? keys[i] : 0;
+  }
+  RowStat st = stat_identity();
   if (wave == 0 && lane < a.splits) {
     const float2 p = a.part_stat[r * a.splits + lane];
     st.mx = p.x;
     st.s = p.y;
   }
-  // A lower bound of the k-th largest from the heads of the lists: the largest 64 / splits keys of every
-  // split (more than k keys in all); its k-th largest keeps a few dozen of the splits * k keys.
   if (tid == 0) {
     sh.thr4[0] = 0;
     sh.cnt = 0;
   }
+  if (m > kRowWG) {  // staged for the bound below
+#pragma unroll
+    for (int q = 0; q < kPer; ++q) {
+      const int i = tid + q * kRowWG;
+      if (i < m) sh.b[i] = mine[q];
+    }
+  }
   __syncthreads();
+  // A lower bound of the k-th largest from the heads of the lists: the largest 64 / splits keys of every
+  // split (more than k keys in all); its k-th largest keeps a few dozen of the splits * k keys.
   if (m > kRowWG && wave == 0) {
     const int per = 64 / a.splits;                 // >= 1: splits <= 64
     const int sp = lane / per, j = lane % per;
-    const uint64_t key = (sp < a.splits && j < k) ? keys[sp * k + j] : 0;
+    const uint64_t key = (sp < a.splits && j < k) ? sh.b[sp * k + j] : 0;
     const int rank = wave_rank(key, 64);
     if (key != 0 && rank == k - 1) sh.thr4[0] = key;
   }
   __syncthreads();
   const uint64_t thr = sh.thr4[0];
-  for (int i = tid; i < m; i += kRowWG) {
-    const uint64_t key = keys[i];
+#pragma unroll
+  for (int q = 0; q < kPer; ++q) {
+    const uint64_t key = mine[q];
     if (key != 0 && key >= thr) sh.a[atomicAdd(&sh.cnt, 1)] = key;
   }
   __syncthreads();
