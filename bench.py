@@ -46,7 +46,8 @@ SETTLE = {"ms": SETTLE_MS}
 CLOCK = {"ms": 400.0}           # GPU-busy time of the clock pass of the matrix-core legs (--clock-ms; 0 = none)
 SETTLE_MAX_LAUNCHES = 2000
 LEGS = ["row", "config1", "ceiling", "fused", "gemm", "config4", "config5", "small", "midsize", "decode", "lora"]
-SUSTAINED = {"tflops": None}    # bf16 MFMA rate of the probe loop on random operands, measured by the `ceiling` leg
+SUSTAINED = {"tflops": None, "with_fill": None, "with_fill_and_fold": None}   # bf16 MFMA rate of the probe loop on random operands, bare and with the
+                                                  # fused kernel's fill requests, measured by the `ceiling` leg
 
 
 def log(*a):
@@ -210,6 +211,9 @@ def mfma_roofline(flop, ms, traffic, kernel, sclk_mhz=None):
     if SUSTAINED["tflops"]:   # what the bare LDS -> MFMA loop reaches on random bf16 operands, same run (`ceiling` leg)
         r["sustained_peak"] = SUSTAINED["tflops"]
         r["frac_of_sustained"] = tf / SUSTAINED["tflops"]
+    if SUSTAINED["with_fill"]:   # the same loop issuing the fused kernel's eight global -> LDS requests per wave and slab
+        r["sustained_peak_with_fill"] = SUSTAINED["with_fill"]
+        r["frac_of_sustained_with_fill"] = tf / SUSTAINED["with_fill"]
     return r
 
 
@@ -405,7 +409,7 @@ def bench_dual(dev, steps, warmup, n=32 * 2048, H=4096):
     return tm
 
 
-def bench_ceiling(dev, steps, warmup, operands="random", with_requests=False):
+def bench_ceiling(dev, steps, warmup, operands="random", with_requests=False, with_fold=False, with_barrier=False):
     """The fused kernel's LDS -> MFMA inner loop alone (tome_probe_mfma_ceiling): one workgroup per CU, operands
     copied into LDS once, no global loads, barriers or epilogue in the loop.  `random`: W rows ~N(0, 0.02^2) and
     token rows ~N(0, 1) as in config 3; `constant`: every operand 1.0."""
@@ -425,7 +429,7 @@ def bench_ceiling(dev, steps, warmup, operands="random", with_requests=False):
     stream = torch.cuda.current_stream(dev).cuda_stream
 
     def step():
-        _lib.check(lib.tome_probe_mfma_ceiling(ops.data_ptr(), n_wg, k_steps, 1 if with_requests else 0, sink.data_ptr(), stream))
+        _lib.check(lib.tome_probe_mfma_ceiling(ops.data_ptr(), n_wg, k_steps, (1 if with_requests else 0) | (2 if with_fold else 0) | (4 if with_barrier else 0), sink.data_ptr(), stream))
     step()
     torch.cuda.synchronize()
     assert torch.isfinite(sink).all()
@@ -660,6 +664,9 @@ def main():
         c = bench_ceiling(dev, K, W, "constant")
         q = bench_ceiling(dev, K, W, "random", with_requests=True)
         SUSTAINED["tflops"] = t["flop"] / (t["ms"] * 1e-3) / 1e12
+        f = bench_ceiling(dev, K, W, "random", with_requests=True, with_fold=True, with_barrier=True)
+        SUSTAINED["with_fill"] = q["flop"] / (q["ms"] * 1e-3) / 1e12
+        SUSTAINED["with_fill_and_fold"] = f["flop"] / (f["ms"] * 1e-3) / 1e12
         legs["mfma_ceiling"] = {
             "value": SUSTAINED["tflops"], "unit": "TFLOP/s", **timing_fields(t), "dtype": "bf16 x bf16 -> f32",
             "config": {"workload": "bare LDS -> MFMA loop of the fused kernel (256x256 workgroup tile, v_mfma_f32_16x16x32_bf16, "
@@ -668,10 +675,14 @@ def main():
                        "constant_operands_tflops": c["flop"] / (c["ms"] * 1e-3) / 1e12,
                        "constant_operands_sclk_mhz": c.get("sclk_mhz"),
                        "random_operands_with_fill_requests_tflops": q["flop"] / (q["ms"] * 1e-3) / 1e12,
-                       "random_operands_with_fill_requests_sclk_mhz": q.get("sclk_mhz")},
+                       "random_operands_with_fill_requests_sclk_mhz": q.get("sclk_mhz"),
+                       "random_operands_with_fill_requests_softmax_fold_every_16_slabs_and_step_barrier_tflops": SUSTAINED["with_fill_and_fold"],
+                       "random_operands_with_fill_requests_softmax_fold_every_16_slabs_and_step_barrier_sclk_mhz": f.get("sclk_mhz")},
             "roofline": mfma_roofline(t["flop"], t["ms"], None, "mfma_ceiling_kernel", t.get("sclk_mhz"))}
         legs["mfma_ceiling"]["roofline"].pop("sustained_peak", None)
         legs["mfma_ceiling"]["roofline"].pop("frac_of_sustained", None)
+        legs["mfma_ceiling"]["roofline"].pop("sustained_peak_with_fill", None)
+        legs["mfma_ceiling"]["roofline"].pop("frac_of_sustained_with_fill", None)
         done("mfma_ceiling")
     if "fused" in only:
         t = bench_fused(dev, K, W)
@@ -681,6 +692,10 @@ def main():
             "config": {"workload": "config 3: fused lm_head + log-softmax, hidden [4096,1024] x W [151936,1024] bf16",
                        "tokens": t["tokens"], "hidden": t["H"], "vocab": V, "temperature": 1.0},
             "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("fused_lmhead_config3"), "fused_lmhead_dma_kernel", t.get("sclk_mhz"))}
+        if SUSTAINED["with_fill_and_fold"]:   # the probe with fill requests, a softmax fold per 16 slabs and the step barrier:
+            r = legs["fused_lmhead"]["roofline"]   # this design at K = 1024 on a memory system that always answers from cache
+            r["design_ceiling"] = SUSTAINED["with_fill_and_fold"]
+            r["frac_of_design_ceiling"] = r["achieved"] / r["design_ceiling"]
         done("fused_lmhead")
     if "gemm" in only:
         t = bench_library_gemm(dev, K, W)

@@ -259,11 +259,15 @@ int tome_lora_merge(const TomeLoraJob* jobs, int64_t n_jobs, void* workspace, si
  * workgroup copies into LDS once - for `steps` 64-wide K slabs: no global loads in the loop, no
  * barrier, no epilogue.  One launch does n_workgroups * steps * 2 * 256 * 256 * 64 FLOP; timing it
  * with random operands gives the bf16 MFMA rate this part sustains under its power limit, which
- * bench.py reports beside the published peak.  With with_requests != 0 every wave also issues the
- * fused kernel's eight 1 KiB global -> LDS requests per slab (re-reading `operands`, which stays in
- * the caches): the cost of the fill apart from the L2 side.  `sink` receives n_workgroups * 512 floats.
+ * bench.py reports beside the published peak.  flags & 1: every wave also issues the fused kernel's
+ * eight 1 KiB global -> LDS requests per slab (re-reading `operands`, which stays in the caches): the
+ * cost of the fill apart from the L2 side.  flags & 2: after every 16 slabs (one vocab tile at
+ * K = 1024; `steps` is rounded down to a multiple) the accumulators are folded with the arithmetic of
+ * the fused kernel's online-softmax epilogue.  flags & 4: the fused kernel's workgroup barrier in
+ * every step.  All three together are that kernel at H = 1024 on a memory system that always answers
+ * from cache.  `sink` receives n_workgroups * 512 floats.
  */
-int tome_probe_mfma_ceiling(const void* operands, int n_workgroups, int steps, int with_requests,
+int tome_probe_mfma_ceiling(const void* operands, int n_workgroups, int steps, int flags,
                             float* sink, void* stream);
 
 #ifdef __cplusplus

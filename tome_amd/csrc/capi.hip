@@ -42,8 +42,7 @@ hipError_t fused_pair_launch(const void* hidden, const void* hidden_ref, const v
                              int64_t hidden_stride, int64_t weight_stride, const int32_t* targets,
                              const int32_t* row_valid, float temperature, float* out_lp, float* out_entropy,
                              float* out_ref_lp, float* out_k3, void* workspace, hipStream_t stream);
-hipError_t mfma_probe_launch(const void* operands, int n_workgroups, int steps, int with_requests, float* sink,
-                             hipStream_t stream);
+hipError_t mfma_probe_launch(const void* operands, int n_workgroups, int steps, int flags, float* sink, hipStream_t stream);
 struct LoraJobHost;
 hipError_t lora_merge_launch(const LoraJobHost* jobs, int n_jobs, void* workspace, hipStream_t stream);
 size_t lora_workspace_bytes(const LoraJobHost* jobs, int n_jobs);
@@ -314,13 +313,11 @@ int tome_grpo_pair(const void* hidden_policy, const void* hidden_ref, const void
                                             static_cast<hipStream_t>(stream)));
 }
 
-int tome_probe_mfma_ceiling(const void* operands, int n_workgroups, int steps, int with_requests, float* sink,
-                            void* stream) {
+int tome_probe_mfma_ceiling(const void* operands, int n_workgroups, int steps, int flags, float* sink, void* stream) {
   if (!operands || !sink) return TOME_E_NULL;
   if (n_workgroups <= 0 || n_workgroups > 65536 || steps <= 0 || steps > (1 << 24)) return TOME_E_SHAPE;
   if (reinterpret_cast<uintptr_t>(operands) % 16 != 0) return TOME_E_ALIGN;
-  return hip_result(tome::mfma_probe_launch(operands, n_workgroups, steps, with_requests, sink,
-                                            static_cast<hipStream_t>(stream)));
+  return hip_result(tome::mfma_probe_launch(operands, n_workgroups, steps, flags, sink, static_cast<hipStream_t>(stream)));
 }
 
 static int check_lora_jobs(const TomeLoraJob* jobs, int64_t n_jobs) {
