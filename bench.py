@@ -21,7 +21,10 @@ host meanwhile reads the engine clock the driver reports (`pp_dpm_sclk` of the d
 smoothed value) every few milliseconds; the median of the samples from the second half of that pass
 is `sclk_mhz`, and these legs price themselves against the published peak scaled to that clock as well
 (`roofline.peak_at_sclk`, `roofline.frac_at_sclk`): the published 2.5 PFLOP/s is 256 CUs x 4096 FLOP per clock at the 2.4 GHz peak engine clock, which the part does not
-hold under a matrix-core load on random operands.
+hold under a matrix-core load on random operands.  The `ceiling` leg times the fused kernel's LDS -> MFMA loop
+alone on random operands (`sustained_peak` in the later matrix-core legs), with the kernel's fill requests
+(`sustained_peak_with_fill`) and with requests, softmax fold and step barrier together (`design_ceiling`
+of the `fused_lmhead` leg: the kernel at config 3 on a memory system that always answers from cache).
 
 Prints ONE JSON line on stdout.  Everything else goes to stderr.
 """
