@@ -48,7 +48,8 @@ SETTLE_MS = 60.0                # untimed GPU-busy time in front of every timed 
 SETTLE = {"ms": SETTLE_MS}
 CLOCK = {"ms": 400.0}           # GPU-busy time of the clock pass of the matrix-core legs (--clock-ms; 0 = none)
 SETTLE_MAX_LAUNCHES = 2000
-LEGS = ["row", "config1", "ceiling", "fused", "gemm", "config4", "config5", "small", "midsize", "decode", "lora"]
+LEGS = ["row", "entry", "config1", "fullmatrix", "ceiling", "fused", "norm", "gemm", "config4", "config5", "pair", "small", "midsize",
+        "decode", "lora"]
 SUSTAINED = {"tflops": None, "with_fill": None, "with_fill_and_fold": None}   # bf16 MFMA rate of the probe loop on random operands, bare and with the
                                                   # fused kernel's fill requests, measured by the `ceiling` leg
 
@@ -432,7 +433,9 @@ def bench_ceiling(dev, steps, warmup, operands="random", with_requests=False, wi
     stream = torch.cuda.current_stream(dev).cuda_stream
 
     def step():
-        _lib.check(lib.tome_probe_mfma_ceiling(ops.data_ptr(), n_wg, k_steps, (1 if with_requests else 0) | (2 if with_fold else 0) | (4 if with_barrier else 0), sink.data_ptr(), stream))
+        _lib.check(lib.tome_probe_mfma_ceiling(ops.data_ptr(), ops.numel() * 2, n_wg, k_steps,
+                                                (1 if with_requests else 0) | (2 if with_fold else 0) | (4 if with_barrier else 0),
+                                                sink.data_ptr(), sink.numel() * 4, stream))
     step()
     torch.cuda.synchronize()
     assert torch.isfinite(sink).all()
@@ -512,6 +515,211 @@ def bench_lora(dev, steps, warmup):
     tm = time_steps(step, steps, warmup)
     tm.update({"bytes": n_bytes, "jobs": len(jobs), "rank": rank})
     return tm
+
+
+def bench_full_matrix(dev, steps, warmup, rows, dtype_name):
+    """tome_full_log_softmax, the drop-in of fused_log_softmax (mlx-impl/model.py:77-89): the whole [rows, V] matrix
+    of log-probs in the input dtype.  Algorithmic bytes 3 * V * sizeof(T) per row (one pass for the row's lse, one
+    to read and one to write the matrix).  The small shape rotates through 16 input / output pairs so that rows come
+    from HBM, not from the last-level cache."""
+    import torch
+    import tome_amd
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    dt = torch.bfloat16 if dtype_name == "bf16" else torch.float32
+    code, esize = (1, 2) if dtype_name == "bf16" else (0, 4)
+    nbuf = 1 if rows * V * esize > (1 << 30) else 16
+    g = torch.Generator(device=dev).manual_seed(21)
+    xs = []
+    for _ in range(nbuf):
+        x = torch.empty((rows, V), device=dev, dtype=dt)
+        for i in range(0, rows, 512):
+            x[i:i + 512] = (torch.randn((min(512, rows - i), V), device=dev, generator=g) * 2.0).to(dt)
+        xs.append(x)
+    outs = [torch.empty_like(xs[0]) for _ in range(nbuf)]
+    row_lse = torch.empty(rows, dtype=torch.float32, device=dev)
+    ws_bytes = lib.tome_row_logprob_workspace(rows, V)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    i = [0]
+
+    def step():
+        k = i[0] % nbuf
+        i[0] += 1
+        _lib.check(lib.tome_full_log_softmax(xs[k].data_ptr(), outs[k].data_ptr(), code, rows, V, V, V, 1.0,
+                                             row_lse.data_ptr(), ws.data_ptr(), ws_bytes, stream))
+    step()
+    torch.cuda.synchronize()
+    sample = torch.arange(0, rows, max(1, rows // 16), device=dev)[:16]     # gate: 16 rows against torch in fp64
+    want = torch.log_softmax(xs[0][sample].double(), dim=-1)
+    tol = 1e-4 if dtype_name == "f32" else 0.0625 + 1e-6                     # bf16 output: one ulp at |x| < 16
+    assert (outs[0][sample].double() - want).abs().max().item() <= tol
+    tm = time_steps(step, steps, warmup)
+    tm.update({"rows": rows, "bytes": 3 * rows * V * esize})
+    return tm
+
+
+def bench_norm_lmhead(dev, steps, warmup, n=4096, H=1024):
+    """tome_norm_lmhead_logprob (mlx-impl/model.py:536-538 + node.py:400-404) at config 3's shape with config 2's
+    padding mask (8 sequences x 512 positions, lengths uniform in [64, 512]): the final RMSNorm is applied to the
+    valid rows only, which are then multiplied.  FLOP counted on valid tokens."""
+    import torch
+    import tome_amd
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    g = torch.Generator(device=dev).manual_seed(808)
+    hidden = (torch.randn((n, H), device=dev, generator=g) * 3.0).to(torch.bfloat16)       # pre-norm states
+    norm_w = (1.0 + 0.1 * torch.randn((H,), device=dev, generator=g)).to(torch.bfloat16)
+    weight = (torch.randn((V, H), device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    targets = torch.randint(0, V, (n,), device=dev, generator=g).to(torch.int32)
+    lens = torch.randint(64, 513, (8,), device=dev, generator=g)
+    valid = (torch.arange(512, device=dev)[None, :] < lens[:, None]).to(torch.int32).reshape(-1).contiguous()
+    n_valid = int(valid.sum().item())
+    lp = torch.empty(n, dtype=torch.float32, device=dev)
+    ws_bytes = lib.tome_norm_lmhead_logprob_workspace(n, H, V)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def step():
+        _lib.check(lib.tome_norm_lmhead_logprob(hidden.data_ptr(), norm_w.data_ptr(), 1e-6, weight.data_ptr(), n, H, V, H, H,
+                                                targets.data_ptr(), valid.data_ptr(), 1.0, lp.data_ptr(), None, None, None,
+                                                ws.data_ptr(), ws_bytes, stream))
+    step()
+    torch.cuda.synchronize()
+    idx = torch.nonzero(valid).view(-1)[:: max(1, n_valid // 64)][:64]      # gate: 64 valid rows against torch
+    x = hidden[idx].float()
+    y = (x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6)).to(torch.bfloat16).float() * norm_w.float()
+    ref = torch.log_softmax(y.to(torch.bfloat16).float() @ weight.float().T, dim=-1)
+    ref = ref[torch.arange(idx.numel(), device=dev), targets[idx].long()]
+    assert (lp[idx] - ref).abs().max().item() < 4e-3 and (lp[valid == 0] == 0).all()
+    tm = time_steps(step, steps, warmup, clock=True)
+    tm.update({"tokens": n, "valid": n_valid, "H": H, "flop": 2.0 * n_valid * H * V})
+    return tm
+
+
+def bench_pair(dev, steps, warmup, n=8192, H=4096):
+    """tome_grpo_pair: the policy + reference pass in the reference's own layout (mlx-impl/node.py:65-66, 443): one
+    hidden-state matrix per model, one shared lm_head.  Outputs lp, ref_lp, k3, entropy."""
+    import torch
+    import tome_amd
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    g = torch.Generator(device=dev).manual_seed(909)
+    h_pol = torch.randn((n, H), device=dev, generator=g).to(torch.bfloat16)
+    h_ref = (h_pol.float() + 0.05 * torch.randn((n, H), device=dev, generator=g)).to(torch.bfloat16)
+    weight = torch.empty((V, H), device=dev, dtype=torch.bfloat16)
+    for i in range(0, V, 16384):
+        m = min(16384, V - i)
+        weight[i:i + m] = (torch.randn((m, H), device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    targets = torch.randint(0, V, (n,), device=dev, generator=g).to(torch.int32)
+    outs = [torch.empty(n, dtype=torch.float32, device=dev) for _ in range(4)]
+    ws_bytes = lib.tome_grpo_pair_workspace(n, H, V, 0)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def step():
+        _lib.check(lib.tome_grpo_pair(h_pol.data_ptr(), h_ref.data_ptr(), None, 0.0, weight.data_ptr(), weight.data_ptr(),
+                                      n, H, V, H, H, targets.data_ptr(), None, 1.0, outs[0].data_ptr(), outs[1].data_ptr(),
+                                      outs[2].data_ptr(), outs[3].data_ptr(), ws.data_ptr(), ws_bytes, stream))
+    step()
+    torch.cuda.synchronize()
+    lp, ref_lp, k3, ent = outs
+    assert torch.isfinite(lp).all() and (lp <= 1e-5).all() and (k3 >= 0).all() and (ent > 0).all()
+    idx = torch.arange(0, n, n // 32, device=dev)[:32]
+    for h, got in ((h_pol, lp), (h_ref, ref_lp)):       # gate: 32 rows of each model against fp32 torch
+        ref = torch.log_softmax(h[idx].float() @ weight.float().T, dim=-1)[torch.arange(32, device=dev), targets[idx].long()]
+        assert (got[idx] - ref).abs().max().item() < 2e-3
+    tm = time_steps(step, steps, warmup, clock=True)
+    tm.update({"tokens": n, "H": H, "flop": 2.0 * 2.0 * n * H * V})
+    return tm
+
+
+def bench_ref_entry(dev, steps, warmup, mode):
+    """The entry itself, RefLogprobServicer.process_ref_logprobs_batched (mlx-impl/node.py:391-461), end to end on the
+    host clock: config 2's batch - 256-token prompts, G = 8 completions of U[64, 512] tokens each - over 32 prompts,
+    i.e. 8 chunks of max_ref_batch_size = 32 sequences per call.  The model is a stub whose output is already
+    resident in HBM (the model's forward is not part of this path): `logits` mode returns bf16 logits
+    [32, max_len, V]; `hidden` mode returns final hidden states [32, max_len, 1024] for the fused lm_head kernel.
+    A step is one call of the entry; it ends with the last chunk's log-probs appended to the Python lists."""
+    import numpy as np
+    import torch
+    import tome_amd
+    from tome_amd.node import Completion, Prompt, PromptRollout
+    from tome_amd.wire import iter_ref_work, scatter_ref_logprobs
+    n_prompts, G, p_len, batch, H = 32, 8, 256, 32, 1024
+    rng = np.random.default_rng(2024)
+    prompts = [Prompt(f"p{i}", rng.integers(0, V, size=p_len).tolist()) for i in range(n_prompts)]
+    comp = [[rng.integers(0, V, size=int(rng.integers(64, 513))).tolist() for _ in range(G)] for _ in range(n_prompts)]
+
+    def fresh_results():
+        return [PromptRollout(f"p{i}", [Completion(tokens=c) for c in comp[i]]) for i in range(n_prompts)]
+    max_len = p_len + 511
+    g = torch.Generator(device=dev).manual_seed(3)
+    if mode == "logits":
+        store = torch.empty(batch * max_len * V, device=dev, dtype=torch.bfloat16)
+        for i in range(0, store.numel(), 1 << 28):
+            store[i:i + (1 << 28)] = (torch.randn((min(1 << 28, store.numel() - i),), device=dev, generator=g) * 3.0).to(torch.bfloat16)
+        width, weight = V, None
+    else:
+        store = torch.randn((batch * max_len * H,), device=dev, generator=g).to(torch.bfloat16)
+        weight = (torch.randn((V, H), device=dev, generator=g) * 0.02).to(torch.bfloat16)
+        width = H
+
+    def model(full_ids, cache=None):                   # output already in HBM: a contiguous [B, L, width] view
+        b, length = full_ids.shape
+        return store[: b * length * width].view(b, length, width), None
+    svc = tome_amd.RefLogprobServicer(model, device=dev, max_ref_batch_size=batch, lm_head_weight=weight)
+
+    # gate on what is timed: the entry's lists against direct kernel calls on the same chunks
+    results = fresh_results()
+    svc.process_ref_logprobs_batched(prompts, results, G, 1.0)
+    chunks = list(iter_ref_work(prompts, fresh_results(), G, batch))
+    n_tokens = sum(c.n_scored for c in chunks)
+    assert svc.last_ref_tokens == n_tokens and all(len(c.ref_log_probs) == len(c.tokens) for r in results for c in r.completions)
+    ch = chunks[1]
+    out, _ = model(torch.from_numpy(ch.ids).to(dev))
+    rows_d, tg_d = torch.from_numpy(ch.scored_rows).to(dev), torch.from_numpy(ch.scored_targets).to(dev)
+    if mode == "logits":
+        direct = tome_amd.token_logprobs_rows(out, rows_d, tg_d, 1.0).lp
+    else:
+        direct = tome_amd.fused_lmhead_logprobs(out.reshape(-1, H).index_select(0, rows_d.long()), weight, tg_d, 1.0).lp
+    p_idx, gi = ch.owners[0]
+    assert np.allclose(results[p_idx].completions[gi].ref_log_probs, direct[: int(ch.cu_lens[1])].cpu().numpy(), atol=0, rtol=0)
+
+    def kernel_pass():                                 # the GPU work of one call, without the entry around it
+        for c, (r, t) in zip(chunks, dev_lists):
+            o, _ = model(torch.empty((c.ids.shape[0], c.ids.shape[1]), dtype=torch.int64, device="meta"))
+            if mode == "logits":
+                tome_amd.token_logprobs_rows(o, r, t, 1.0)
+            else:
+                tome_amd.fused_lmhead_logprobs(o.reshape(-1, H).index_select(0, r.long()), weight, t, 1.0)
+    dev_lists = [(torch.from_numpy(c.scored_rows).to(dev), torch.from_numpy(c.scored_targets).to(dev)) for c in chunks]
+    kt = time_steps(kernel_pass, steps, warmup)
+
+    def host_pass():                                   # the host bookkeeping of one call, without the GPU
+        res = fresh_results()
+        t0 = time.perf_counter()
+        for c in iter_ref_work(prompts, res, G, batch):
+            scatter_ref_logprobs(c, np.zeros(c.n_scored, dtype=np.float32), res)
+        return time.perf_counter() - t0
+    host_s = sorted(host_pass() for _ in range(max(5, steps)))
+
+    for _ in range(warmup):
+        svc.process_ref_logprobs_batched(prompts, fresh_results(), G, 1.0)
+    walls = []
+    for _ in range(steps):
+        res = fresh_results()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        svc.process_ref_logprobs_batched(prompts, res, G, 1.0)
+        walls.append((time.perf_counter() - t0) * 1e3)
+    mean_ms = sum(walls) / len(walls)
+    walls.sort()
+    return {"ms": mean_ms, "median_ms": walls[len(walls) // 2], "min_ms": walls[0], "settle_launches": 0,
+            "tokens": n_tokens, "chunks": len(chunks), "sequences": n_prompts * G,
+            "kernel_ms": kt["ms"], "host_us_per_chunk": host_s[len(host_s) // 2] * 1e6 / len(chunks),
+            "bytes": n_tokens * V * 2 if mode == "logits" else None,
+            "flop": 2.0 * n_tokens * H * V if mode == "hidden" else None}
 
 
 # ---- CPU baseline -------------------------------------------------------------------------------------
@@ -652,6 +860,28 @@ def main():
                 "roofline": hbm_roofline(row["bytes_all"], t["ms"], traffic_of("row_logprob_config2_all_rows"),
                                          "row_logprob_kernel<bf16>")}
             done("all_rows")
+    if "entry" in only:
+        for mode in ("logits", "hidden"):
+            t = bench_ref_entry(dev, K, W, mode)
+            name = "ref_entry" if mode == "logits" else "ref_entry_hidden_mode"
+            what = ("the stub model's bf16 logits [32, max_len, 151936] are resident in HBM; tome_row_logprob_rows scores the completion rows"
+                    if mode == "logits" else
+                    "the stub model returns final hidden states [32, max_len, 1024]; the completion rows go through the fused lm_head kernel")
+            roof = (hbm_roofline(t["bytes"], t["kernel_ms"], None, "row_logprob_kernel<bf16> over the scored rows, 8 launches") if mode == "logits"
+                    else mfma_roofline(t["flop"], t["kernel_ms"], None, "fused_lmhead_dma_kernel, 8 launches"))
+            roof["note"] = "priced on kernel_ms (the same launches without the entry around them), not on ms_per_step"
+            legs[name] = {
+                "value": t["tokens"] / (t["ms"] * 1e-3), "unit": "token-logprobs/s at the entry (host clock, lists filled)",
+                **timing_fields(t), "dtype": "f32", "input_dtype": "bf16",
+                "config": {"workload": "RefLogprobServicer.process_ref_logprobs_batched (node.py:391-461) on config 2's batch: 32 prompts of 256 "
+                                       "tokens x G=8 completions of U[64,512] tokens, max_ref_batch_size 32 (8 chunks per call); " + what,
+                           "sequences": t["sequences"], "chunks": t["chunks"], "scored_tokens": t["tokens"], "vocab": V},
+                "kernel_ms": t["kernel_ms"], "kernel_share_of_wall": t["kernel_ms"] / t["ms"],
+                "host_us_per_chunk": t["host_us_per_chunk"], "wall_us_per_chunk": t["ms"] * 1e3 / t["chunks"],
+                "roofline": roof}
+            log(f"{name}: {t['ms']:.2f} ms per call ({t['chunks']} chunks, {t['tokens']} tokens), kernels {t['kernel_ms']:.2f} ms "
+                f"= {t['kernel_ms'] / t['ms']:.2f} of the wall time, host {t['host_us_per_chunk']:.0f} us per chunk")
+            torch.cuda.empty_cache()
     if "config1" in only:
         t = bench_config1(dev, K, W)
         legs["config1_row"] = {
@@ -662,6 +892,24 @@ def main():
             "roofline": hbm_roofline(t["bytes"], t["ms"], traffic_of("row_logprob_config1"),
                                      "row_logprob_kernel<f32> (8 workgroups per row) + row_combine_kernel")}
         done("config1_row")
+    if "fullmatrix" in only:
+        shapes = {}
+        for rows, dn in ((4096, "bf16"), (64, "f32")):
+            t = bench_full_matrix(dev, K, W, rows, dn)
+            shapes[f"{rows}x{V}_{dn}"] = {**timing_fields(t), "roofline": hbm_roofline(
+                t["bytes"], t["ms"], traffic_of(f"full_log_softmax_{rows}rows_{dn}"),
+                "row_logprob_kernel (lse) + full_log_softmax_kernel")}
+            log(f"full matrix {rows} x {V} {dn}: {t['ms'] * 1e3:.1f} us, {shapes[f'{rows}x{V}_{dn}']['roofline']['frac']:.3f} of HBM peak")
+            torch.cuda.empty_cache()
+        big = shapes[f"4096x{V}_bf16"]
+        legs["full_log_softmax"] = {
+            "value": 4096 * V / (big["ms_per_step"] * 1e-3), "unit": "log-probs written/s (4096 x 151936 bf16)",
+            **{k: big[k] for k in ("ms_per_step", "median_ms", "min_ms", "settle_launches")}, "dtype": "f32", "input_dtype": "bf16",
+            "config": {"workload": "tome_full_log_softmax, the drop-in of fused_log_softmax (model.py:77-89): the whole log-prob matrix in the "
+                                   "input dtype; [4096, 151936] bf16 and [64, 151936] fp32 (16 rotating buffers); algorithmic bytes 3 V sizeof(T) per row",
+                       "shapes": shapes},
+            "roofline": big["roofline"]}
+        done("full_log_softmax")
     if "ceiling" in only:
         t = bench_ceiling(dev, K, W, "random")
         c = bench_ceiling(dev, K, W, "constant")
@@ -700,6 +948,16 @@ def main():
             r["design_ceiling"] = SUSTAINED["with_fill_and_fold"]
             r["frac_of_design_ceiling"] = r["achieved"] / r["design_ceiling"]
         done("fused_lmhead")
+    if "norm" in only:
+        t = bench_norm_lmhead(dev, K, W)
+        legs["norm_lmhead"] = {
+            "value": t["valid"] / (t["ms"] * 1e-3), "unit": "token-logprobs/s", **timing_fields(t), "dtype": "bf16 x bf16 -> f32",
+            "config": {"workload": "tome_norm_lmhead_logprob (model.py:536-538): final RMSNorm + lm_head + log-softmax, pre-norm hidden "
+                                   "[8x512, 1024] x W [151936, 1024] bf16 with config 2's padding mask (lengths~U[64,512]); FLOP on valid tokens",
+                       "tokens": t["tokens"], "valid_tokens": t["valid"], "hidden": t["H"], "vocab": V},
+            "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("norm_lmhead_config3_masked"),
+                                      "compact_rows + rmsnorm_rows + fused_lmhead_dma_kernel + combine", t.get("sclk_mhz"))}
+        done("norm_lmhead")
     if "gemm" in only:
         t = bench_library_gemm(dev, K, W)
         legs["library_gemm_config3"] = {
@@ -729,6 +987,17 @@ def main():
             "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("grpo_dual_config5"),
                                       "fused_lmhead_dma_kernel (two sweeps) + fused_combine_kernel", t.get("sclk_mhz"))}
         done("config5_grpo_dual")
+    if "pair" in only:
+        t = bench_pair(dev, K, W)
+        legs["grpo_pair"] = {
+            "value": t["tokens"] / (t["ms"] * 1e-3), "unit": "tokens/s (lp, ref_lp, k3, entropy each)", **timing_fields(t),
+            "dtype": "bf16 x bf16 -> f32",
+            "config": {"workload": "tome_grpo_pair (node.py:65-66, 443): policy and reference hidden states [8192, 4096] each, one shared "
+                                   "W [151936, 4096] bf16; outputs lp, ref_lp, k3, entropy",
+                       "tokens": t["tokens"], "hidden": t["H"], "vocab": V, "temperature": 1.0},
+            "roofline": mfma_roofline(t["flop"], t["ms"], traffic_of("grpo_pair_8192x4096"),
+                                      "fused_lmhead_dma_kernel (two sweeps) + fused_combine_kernel", t.get("sclk_mhz"))}
+        done("grpo_pair")
     if "small" in only:
         t = bench_fused(dev, K, W, n=64)
         legs["fused_lmhead_decode_batch"] = {

@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define TOME_ABI_VERSION 2
+#define TOME_ABI_VERSION 3
 
 enum { TOME_F32 = 0, TOME_BF16 = 1 };
 
@@ -96,7 +96,8 @@ int tome_row_logprob_rows(const void* logits, int dtype, int64_t n_rows, int64_t
  * a fixed memory plan, harnesses that forbid hipMalloc.  Same arguments, kernels and results
  * as tome_row_logprob, minus the workspace: the per-(row, split) partials of small batches
  * go to a fixed 64 KiB array inside the library's code object (one copy per GPU, held until
- * the process ends).  The call allocates and frees nothing.  A call whose partials would not
+ * the process ends).  The call allocates and frees nothing and, after the first call on a GPU, takes no
+ * lock.  A call whose partials would not
  * fit returns TOME_E_SCRATCH before any launch (with the library's split rule - fewer than
  * 512 rows are split so that about 512 workgroups run - no shape needs more than 16 KiB).
  * All calls on one GPU share the array: calls that overlap in time on the same GPU (different
@@ -108,6 +109,11 @@ int tome_row_logprob_noalloc(const void* logits, int dtype, int64_t rows, int64_
                              const int32_t* targets, const int32_t* row_valid, float temperature,
                              float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
                              void* stream);
+/* Testing hook, no counterpart in the reference: lowers the number of bytes of that array a call may use
+ * (0 or anything above 64 KiB restores the whole array) and returns the limit now in force, so that the
+ * TOME_E_SCRATCH path, which no shape reaches with the whole array, can be exercised.  Process-wide; not for
+ * production callers. */
+size_t tome_row_logprob_noalloc_limit(size_t bytes);
 
 /* ---- Decode-step sampler on the same logits pass -----------------------------------
  * Replaces, for a batch of decode rows, _sample_token(logits, temperature, top_k=20)
@@ -265,10 +271,13 @@ int tome_lora_merge(const TomeLoraJob* jobs, int64_t n_jobs, void* workspace, si
  * K = 1024; `steps` is rounded down to a multiple) the accumulators are folded with the arithmetic of
  * the fused kernel's online-softmax epilogue.  flags & 4: the fused kernel's workgroup barrier in
  * every step.  All three together are that kernel at H = 1024 on a memory system that always answers
- * from cache.  `sink` receives n_workgroups * 512 floats.
+ * from cache.  `operands` must hold at least 64 KiB (`operand_bytes`) and `sink` receives
+ * n_workgroups * 512 floats (`sink_bytes` must cover them); smaller buffers, n_workgroups outside
+ * 1..4096, steps outside 1..65536 and flags outside 0..7 return TOME_E_SHAPE before any launch (one
+ * launch is at most a few hundred milliseconds of GPU time).
  */
-int tome_probe_mfma_ceiling(const void* operands, int n_workgroups, int steps, int flags,
-                            float* sink, void* stream);
+int tome_probe_mfma_ceiling(const void* operands, size_t operand_bytes, int n_workgroups, int steps,
+                            int flags, float* sink, size_t sink_bytes, void* stream);
 
 #ifdef __cplusplus
 }

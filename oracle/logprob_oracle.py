@@ -155,13 +155,18 @@ def full_log_softmax64(x: np.ndarray, temperature: float = 1.0) -> np.ndarray:
 
 
 def entropy_rows(x: np.ndarray, temperature: float = 1.0) -> np.ndarray:
-    """H[r] = lse - sum_j p_j z_j with z = x/T, p = softmax(z).  Not in the reference."""
+    """H[r] = lse - sum_j p_j z_j with z = x/T, p = softmax(z).  Not in the reference.
+
+    Entries of -inf (a masked vocabulary) have p_j = 0 and contribute nothing (0 log 0 = 0).
+    """
     z = _scaled(x, temperature)
     m = z.max(axis=-1, keepdims=True)
-    e = np.exp(z - m)
+    with np.errstate(invalid="ignore"):
+        e = np.exp(z - m)
+        ez = np.where(np.isneginf(z), 0.0, e * z)
     s = e.sum(axis=-1)
     lse = m[..., 0] + np.log(s)
-    return lse - (e * z).sum(axis=-1) / s
+    return lse - ez.sum(axis=-1) / s
 
 
 def argmax_rows(x: np.ndarray) -> np.ndarray:

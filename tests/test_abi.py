@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(tome_amd.lib_path())
     for name in declared_functions():
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
-    assert tome_amd.load_library().tome_abi_version() == 2
+    assert tome_amd.load_library().tome_abi_version() == 3
 
 
 def test_header_cites_reference_for_each_entry_point():
@@ -80,6 +80,16 @@ def test_argument_checks_run_on_host():
     assert na(dtype=7) == -2 and na(V=0) == -3 and na(stride=63) == -3 and na(T=0.0) == -5
     assert na(logits=None) == -1 and na(targets=None) == -1 and na(lp=None) == -1 and na(rows=0) == 0
     assert na(logits=P + 1) == -6
+    # TOME_E_SCRATCH: no shape needs more than 16 KiB of the 64 KiB array, so the limit is lowered to reach the path
+    assert lib.tome_row_logprob_noalloc_limit(4096) == 4096
+    try:
+        assert na(rows=300, V=151936, stride=151936) == -8           # 300 rows x 2 splits x 16 B of partials > 4096
+        assert na(rows=300, V=151936, stride=151936, logits=None) == -1   # argument checks still come first
+        with pytest.raises(ValueError, match="scratch"):
+            _lib.check(-8)
+    finally:
+        assert lib.tome_row_logprob_noalloc_limit(0) == 64 * 1024   # 0 restores the whole array
+    assert lib.tome_row_logprob_noalloc_limit(1 << 30) == 64 * 1024  # and nothing raises it beyond the array
     rl = lambda **k: lib.tome_row_logprob_rows(k.get("logits", P), k.get("dtype", 1), k.get("rows", 4), k.get("V", 64),
                                                k.get("stride", 64), k.get("idx", P), k.get("n", 3), k.get("targets", P),
                                                k.get("T", 1.0), k.get("lp", P), None, None, None, None, 0, None)
@@ -116,6 +126,13 @@ def test_argument_checks_run_on_host():
     assert pair() == -4
     assert lib.tome_grpo_pair_workspace(4096, 1024, 151936, 0) == lib.tome_grpo_dual_workspace(4096, 1024, 151936)
     assert lib.tome_grpo_pair_workspace(4096, 1024, 151936, 1) >= lib.tome_grpo_dual_workspace(4096, 1024, 151936) + 2 * 4096 * 1024 * 2
+
+    probe = lambda **k: lib.tome_probe_mfma_ceiling(k.get("ops", P), k.get("ob", 65536), k.get("wg", 256), k.get("steps", 16),
+                                                    k.get("flags", 0), k.get("sink", P), k.get("sb", 256 * 512 * 4), None)
+    assert probe(ops=None) == -1 and probe(sink=None) == -1 and probe(ops=P + 4) == -6
+    assert probe(ob=65535) == -3 and probe(sb=256 * 512 * 4 - 1) == -3          # buffers smaller than the kernel touches
+    assert probe(wg=0) == -3 and probe(wg=4097) == -3 and probe(steps=0) == -3 and probe(steps=65537) == -3
+    assert probe(flags=8) == -3 and probe(flags=-1) == -3
 
     def merge(**k):
         j = _lib.TomeLoraJob()

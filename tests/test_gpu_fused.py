@@ -333,3 +333,40 @@ def test_fused_all_masked_and_single_valid_row(dev, n, H):
     assert abs(r.lp[n // 2].item() - want["lp"][0]) < TOL and (r.lp[one == 0] == 0).all()
     d = tome_amd.grpo_dual_logprobs(h, w, w, tt, 1.0, row_valid=one)
     assert d.k3[n // 2].item() == 0.0 and (d.k3[one == 0] == 0).all()
+
+
+@pytest.mark.parametrize("which,kind,n", [("weight", "dma", 200), ("weight", "dma", 100), ("weight", "small", 32),
+                                          ("hidden", "dma", 300)])
+def test_fused_matrices_of_4_gib_and_more(dev, which, kind, n):
+    """The LDS-DMA and streaming kernels address both matrices with 64-bit offsets, so a weight (or hidden-state)
+    matrix whose extent V * weight_stride * 2 (n * hidden_stride * 2) reaches 2^32 bytes is accepted; only the
+    generic kernel refuses it.  A padded row stride makes the extent 4.3 GB while 512 columns are used.  Targets
+    and a planted maximum sit in the LAST rows, which lie beyond the 4 GiB mark."""
+    H, V = 512, 40000
+    lib = tome_amd.load_library()
+    rng = np.random.default_rng(n)
+    stride = 53760 if which == "weight" else 512                      # 40000 * 53760 * 2 = 4.30e9 >= 2^32
+    hstride = 512 if which == "weight" else 7158336                   # 300 * 7158336 * 2 = 4.29e9 >= 2^32
+    assert (V * stride * 2 >= 1 << 32) != (n * hstride * 2 >= 1 << 32)
+    w_store = torch.empty((V, stride), dtype=torch.bfloat16, device=dev)
+    w = w_store[:, :H]
+    w.copy_(torch.from_numpy((rng.standard_normal((V, H)) * 0.05).astype(np.float32)).to(dev))
+    h_store = torch.empty((n, hstride), dtype=torch.bfloat16, device=dev)
+    h = h_store[:, :H]
+    h.copy_(torch.from_numpy(rng.standard_normal((n, H)).astype(np.float32)).to(dev))
+    t = rng.integers(V - 300, V, size=n).astype(np.int32)            # rows past the 4 GiB mark of the weight matrix
+    w[V - 3] = 0.5 * torch.sign(h[n - 1].float()).to(torch.bfloat16)  # token n-1 (past the mark of the hidden matrix): row V-3 wins
+    lib.tome_select_fused_kernel({"dma": 1, "small": -1}[kind])
+    try:
+        r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 1.0, want_lse=True, want_argmax=True)
+        torch.cuda.synchronize()
+        lib.tome_select_fused_kernel(0)                              # the generic kernel keeps refusing the shape
+        with pytest.raises(ValueError):
+            tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 1.0)
+    finally:
+        lib.tome_select_fused_kernel(-1)
+    want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(w), t, 1.0)
+    np.testing.assert_allclose(r.lp.cpu().numpy(), want["lp"], atol=TOL, rtol=0)
+    np.testing.assert_allclose(r.lse.cpu().numpy(), want["lse"], atol=TOL, rtol=0)
+    assert r.argmax.cpu().numpy()[n - 1] == V - 3 == want["argmax"][n - 1]
+    check_argmax(h, w, r.argmax.cpu().numpy(), want)

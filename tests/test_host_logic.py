@@ -168,3 +168,45 @@ def test_servicer_is_async_like_the_reference():
     # nothing to score: must finish without calling the model or the GPU
     asyncio.run(s._process_ref_logprobs_batched([Prompt("p", [1])], [PromptRollout("p", [Completion()])], 1))
     assert s.last_ref_tokens == 0
+
+
+@pytest.mark.parametrize("loop", ["rollout", "judge"])
+def test_decode_loops_refuse_a_row_without_a_token(monkeypatch, loop):
+    """The sampler answers -1 for an active row with no logit above -inf.  The decode loops must not feed that id
+    to the next model step (an out-of-range embedding index on the device); they raise, naming the row.  The
+    sampler is stubbed here (greedy over CPU tensors) so that the bookkeeping runs without a GPU."""
+    from tome_amd import decode as dec
+    from tome_amd.logprob import SampledTokens
+
+    def stub_sampler(logits, temperature, top_k, *, uniforms=None, row_valid=None):
+        best, tok = logits.max(dim=-1)
+        tok = torch.where(torch.isneginf(best), torch.full_like(tok, -1), tok).to(torch.int32)
+        if row_valid is not None:
+            tok = torch.where(row_valid != 0, tok, torch.full_like(tok, -1))
+        lp = torch.zeros(tok.shape, dtype=torch.float32)
+        return SampledTokens(tok, lp, tok, None, None)
+
+    monkeypatch.setattr(dec, "sample_tokens", stub_sampler)
+    V, B = 16, 3
+    first = torch.zeros(B, V)
+    first[:, 4] = 1.0
+    seen = []
+
+    def model_step(tokens):
+        seen.append(tokens.tolist())
+        out = torch.zeros(B, V)
+        out[:, 5] = 1.0
+        if len(seen) == 2:
+            out[1] = float("-inf")                  # row 1 diverges at the second step
+        return out
+
+    run = (lambda: dec.rollout_decode(model_step, first, 1, 0.0, 6, 9)) if loop == "rollout" else \
+          (lambda: dec.judge_decode(model_step, first, 0.0, 6, 9))
+    with pytest.raises(RuntimeError, match=r"rows \[1\]"):
+        run()
+    assert all(t >= 0 for step in seen for t in step)   # no negative id ever reached the model
+    # a masked (finished) row's -1 is not an error: eos = 5 ends every row at the first loop step
+    seen.clear()
+    done = dec.rollout_decode(lambda t: model_step(t), first, 1, 0.0, 6, 5) if loop == "rollout" else \
+        dec.judge_decode(lambda t: model_step(t), first, 0.0, 6, 5)
+    assert [d["tokens"] for d in done] == ([[4, 5]] * B if loop == "rollout" else [[4]] * B)

@@ -365,3 +365,28 @@ def test_decode_loops_use_the_sampler_with_temperature():
         for row, tok, lp in zip(rows, s["tokens"], s["log_probs"]):
             assert tok in np.argsort(-row)[:5]
             np.testing.assert_allclose(lp, scipy.special.log_softmax(row / 0.8)[tok], atol=1e-12)
+
+
+def test_masked_vocabulary_rows_against_scipy_and_torch():
+    """Rows with -inf entries (a masked vocabulary): the closed forms reduce to those of the kept entries, checked
+    against scipy / torch.float64 on the same rows and against the oracle on the row with the masked entries removed."""
+    import torch
+    rng = np.random.default_rng(41)
+    V, T = 3000, 0.8
+    x = (rng.standard_normal((5, V)) * 3).astype(np.float32)
+    keep = rng.random((5, V)) > 0.4
+    keep[:, 7] = True
+    xm = np.where(keep, x, -np.inf).astype(np.float32)
+    t = np.array([7, 7, 7, 7, int(np.flatnonzero(~keep[4])[0])])        # the last target is a masked id
+    z = xm.astype(np.float64) / T
+    np.testing.assert_allclose(oracle.lse_rows(xm, T), scipy.special.logsumexp(z, axis=-1), atol=1e-12)
+    tl = torch.log_softmax(torch.from_numpy(z), dim=-1).numpy()
+    got = oracle.logprob_rows(xm, t, T)
+    np.testing.assert_allclose(got[:4], tl[np.arange(4), t[:4]], atol=1e-12)
+    assert got[4] == -np.inf
+    for r in range(5):
+        dense = x[r][keep[r]][None, :]
+        np.testing.assert_allclose(oracle.lse_rows(xm[r:r + 1], T), oracle.lse_rows(dense, T), atol=1e-12)
+        np.testing.assert_allclose(oracle.entropy_rows(xm[r:r + 1], T), oracle.entropy_rows(dense, T), atol=1e-12)
+        assert oracle.argmax_rows(xm[r:r + 1])[0] == np.flatnonzero(keep[r])[np.argmax(x[r][keep[r]])]
+    np.testing.assert_allclose(oracle.entropy_rows(xm, T), scipy.stats.entropy(np.exp(tl), axis=-1), atol=1e-10)

@@ -73,3 +73,43 @@ def test_noalloc_checked_against_the_oracle(dev):
     want = oracle.logprob_rows(x.cpu().numpy(), t.cpu().numpy(), 1.0)
     assert np.abs(lp.cpu().numpy() - want).max() < 1e-4     # fp32 logits: 1e-4 abs
     assert (am.cpu().numpy() == oracle.argmax_rows(x.cpu().numpy())).all()
+
+
+def test_noalloc_replays_from_a_hip_graph(dev):
+    """The callers this entry point is for include code under HIP graph capture: after one eager call (which looks
+    the scratch address up, outside any capture) the call is captured and replayed on changing inputs; every replay
+    must equal the eager call on the same inputs bit for bit, with unrelated eager work between the replays."""
+    import torch
+    import tome_amd
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    rows, V = 48, 60000
+    g = torch.Generator(device=dev).manual_seed(5)
+    x = torch.zeros((rows, V), dtype=torch.float32, device=dev)
+    t = torch.zeros(rows, dtype=torch.int32, device=dev)
+    outs = {k: (torch.empty(rows, dtype=torch.float32, device=dev), torch.empty(rows, dtype=torch.int32, device=dev))
+            for k in ("graph", "eager")}
+
+    def call(which, stream):
+        lp, am = outs[which]
+        _lib.check(lib.tome_row_logprob_noalloc(x.data_ptr(), 0, rows, V, V, t.data_ptr(), None, 0.8, lp.data_ptr(), None,
+                                                None, am.data_ptr(), stream))
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        call("graph", side.cuda_stream)                                   # warm-up: resolves the scratch address
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        call("graph", torch.cuda.current_stream(dev).cuda_stream)
+    for it in range(3):
+        x.copy_(torch.randn((rows, V), device=dev, generator=g) * (1.0 + it))
+        t.copy_(torch.randint(0, V, (rows,), device=dev, generator=g).to(torch.int32))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        call("eager", torch.cuda.current_stream(dev).cuda_stream)
+        torch.cuda.synchronize()
+        assert torch.equal(outs["graph"][0], outs["eager"][0]) and torch.equal(outs["graph"][1], outs["eager"][1])
+        assert torch.isfinite(outs["graph"][0]).all()
+        (x[:8] @ x[:8].T).sum().item()                                    # unrelated eager work between replays

@@ -10,7 +10,7 @@ _LIB_PATH = os.path.join(_PKG_DIR, "libtome_logprob.so")
 _lib: ctypes.CDLL | None = None
 
 TOME_F32, TOME_BF16 = 0, 1
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # name -> (restype, argtypes); must list every function the header declares.
 SIGNATURES = {
@@ -24,6 +24,7 @@ SIGNATURES = {
                                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "tome_row_logprob_noalloc": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "tome_row_logprob_noalloc_limit": (c_size_t, [c_size_t]),
     "tome_row_sample_workspace": (c_size_t, [c_int, c_int64, c_int64, c_int]),
     "tome_row_sample": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float, c_int,
                                 c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
@@ -47,7 +48,7 @@ SIGNATURES = {
     "tome_grpo_pair": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                c_int64, c_int64, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_size_t, c_void_p]),
-    "tome_probe_mfma_ceiling": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "tome_probe_mfma_ceiling": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "tome_lora_merge_workspace": (c_size_t, [c_void_p, c_int64]),
     "tome_lora_merge": (c_int, [c_void_p, c_int64, c_void_p, c_size_t, c_void_p]),
 }

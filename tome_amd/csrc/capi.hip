@@ -16,6 +16,7 @@ hipError_t row_logprob_launch_rows(const void* logits, int dtype, int64_t n_rows
                                    float temperature, float* out_lp, float* out_lse, float* out_entropy,
                                    int32_t* out_argmax, void* workspace, hipStream_t stream);
 int row_splits_for(int64_t rows, int64_t V, int vec);
+size_t row_scratch_set_limit(size_t bytes);
 hipError_t row_logprob_noalloc_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
                                       const int32_t* targets, const int32_t* row_valid, float temperature,
                                       float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
@@ -158,6 +159,8 @@ int tome_row_logprob_noalloc(const void* logits, int dtype, int64_t rows, int64_
   if (too_big) return TOME_E_SCRATCH;
   return hip_result(e);
 }
+
+size_t tome_row_logprob_noalloc_limit(size_t bytes) { return tome::row_scratch_set_limit(bytes); }
 
 size_t tome_row_sample_workspace(int dtype, int64_t rows, int64_t V, int top_k) {
   if (rows <= 0 || V <= 0 || top_k < 1 || top_k > 32) return 0;
@@ -313,9 +316,13 @@ int tome_grpo_pair(const void* hidden_policy, const void* hidden_ref, const void
                                             static_cast<hipStream_t>(stream)));
 }
 
-int tome_probe_mfma_ceiling(const void* operands, int n_workgroups, int steps, int flags, float* sink, void* stream) {
+int tome_probe_mfma_ceiling(const void* operands, size_t operand_bytes, int n_workgroups, int steps, int flags,
+                            float* sink, size_t sink_bytes, void* stream) {
   if (!operands || !sink) return TOME_E_NULL;
-  if (n_workgroups <= 0 || n_workgroups > 65536 || steps <= 0 || steps > (1 << 24)) return TOME_E_SHAPE;
+  // Bounded so that one call cannot occupy the GPU for long: 4096 workgroups x 65536 slabs is a few hundred ms.
+  if (n_workgroups <= 0 || n_workgroups > 4096 || steps <= 0 || steps > (1 << 16) || flags < 0 || flags > 7)
+    return TOME_E_SHAPE;
+  if (operand_bytes < (size_t)64 * 1024 || sink_bytes < (size_t)n_workgroups * 512 * sizeof(float)) return TOME_E_SHAPE;
   if (reinterpret_cast<uintptr_t>(operands) % 16 != 0) return TOME_E_ALIGN;
   return hip_result(tome::mfma_probe_launch(operands, n_workgroups, steps, flags, sink, static_cast<hipStream_t>(stream)));
 }

@@ -13,6 +13,7 @@
 // results do not depend on scheduling).
 #include "row_common.hpp"
 
+#include <atomic>
 #include <mutex>
 
 namespace tome {
@@ -289,26 +290,37 @@ constexpr size_t kRowScratchBytes = 64 * 1024;
 static __device__ __align__(256) unsigned char scratch[kRowScratchBytes];
 
 constexpr int kMaxDevices = 64;
-static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch`, per device ordinal
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];  // device address of `scratch`, per device ordinal
 static std::mutex g_scratch_mutex;
+// Bytes of the array a call may use: the whole array, unless a test lowered it to reach the error path.
+static std::atomic<size_t> g_scratch_limit{kRowScratchBytes};
 
 size_t row_scratch_capacity() { return kRowScratchBytes; }
+size_t row_scratch_set_limit(size_t bytes) {
+  const size_t lim = (bytes == 0 || bytes > kRowScratchBytes) ? kRowScratchBytes : bytes;
+  g_scratch_limit.store(lim, std::memory_order_relaxed);
+  return lim;
+}
 
 // Address of this device's copy of the scratch array; resolved once per device, with that device current.
+// After that first call the address is read without taking the lock.
 static hipError_t row_scratch_for_current_device(void** out) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
-  std::lock_guard<std::mutex> lock(g_scratch_mutex);
-  if (!g_scratch_ptr[dev]) {
-    void* p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    if (e != hipSuccess) return e;
-    if (!p) return hipErrorInvalidSymbol;
-    g_scratch_ptr[dev] = p;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+    if (!p) {
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess) return e;
+      if (!p) return hipErrorInvalidSymbol;
+      g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
   }
-  *out = g_scratch_ptr[dev];
+  *out = p;
   return hipSuccess;
 }
 
@@ -326,7 +338,7 @@ hipError_t row_logprob_noalloc_launch(const void* logits, int dtype, int64_t row
                                       const int32_t* targets, const int32_t* row_valid, float temperature,
                                       float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
                                       bool* too_big, hipStream_t stream) {
-  *too_big = row_partials_bytes(logits, dtype, rows, V, row_stride) > kRowScratchBytes;
+  *too_big = row_partials_bytes(logits, dtype, rows, V, row_stride) > g_scratch_limit.load(std::memory_order_relaxed);
   if (*too_big) return hipSuccess;
   void* ptr = nullptr;
   const hipError_t e = row_scratch_for_current_device(&ptr);

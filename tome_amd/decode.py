@@ -29,8 +29,13 @@ def _uniforms(source, step: int, rows: int, dev: torch.device, generator) -> Opt
     return torch.as_tensor(u, dtype=torch.float32, device=dev).reshape(rows)
 
 
-def _step(logits: torch.Tensor, temperature: float, top_k: int, uniforms, row_valid: Optional[torch.Tensor]):
-    """Sample every active row; returns the device token ids and, after ONE copy, the host (token, lp) arrays."""
+def _step(logits: torch.Tensor, temperature: float, top_k: int, uniforms, row_valid: Optional[torch.Tensor],
+          active: Optional[np.ndarray] = None):
+    """Sample every active row; returns the device token ids and, after ONE copy, the host (token, lp) arrays.
+
+    ``active`` is the host copy of ``row_valid`` (None = every row).  The sampler answers -1 for a row it was asked
+    to draw from that holds no logit above -inf (a model that has diverged); such an id must not reach the next
+    ``model_step`` as an embedding index, so it is an error here, naming the rows."""
     out = sample_tokens(logits, temperature, top_k, uniforms=uniforms if temperature > 0 else None, row_valid=row_valid)
     n = out.token.numel()
     tok, lp = out.token.reshape(-1), out.lp.reshape(-1)
@@ -39,7 +44,12 @@ def _step(logits: torch.Tensor, temperature: float, top_k: int, uniforms, row_va
     else:
         both = torch.cat([tok, lp.view(torch.int32)])
     host = both.cpu().numpy()                                                  # one sync, one copy
-    return out.token, host[:n].astype(np.int64), host[n:].view(np.float32)
+    tok_h = host[:n].astype(np.int64)
+    bad = tok_h < 0 if active is None else (tok_h < 0) & active
+    if bad.any():
+        raise RuntimeError(f"decode step: no token could be drawn for rows {np.flatnonzero(bad).tolist()} "
+                           "(no logit above -inf); the model's logits are degenerate")
+    return out.token, tok_h, host[n:].view(np.float32)
 
 
 def _mask_to_device(active: np.ndarray, dev: torch.device) -> torch.Tensor:
@@ -90,7 +100,7 @@ def rollout_decode(model_step: Callable[[torch.Tensor], torch.Tensor], last_logi
             inputs = torch.where(rv_dev != 0, inputs, eos_dev)                 # node.py:593-595
         logits = model_step(inputs)
         dev_tok, tok, lp = _step(logits, temperature, top_k, _uniforms(uniform_source, step + 1, total, dev, generator),
-                                 rv_dev)
+                                 rv_dev, ~finished)
         act = ~finished
         rows = np.nonzero(act)[0]
         toks[rows, lens[rows]] = tok[rows]                                     # node.py:604-605
@@ -132,7 +142,8 @@ def judge_decode(model_step: Callable[[torch.Tensor], torch.Tensor], first_logit
         if rv_dev is not None:
             inputs = torch.where(rv_dev != 0, inputs, zero_dev)                # node.py:350
         logits = model_step(inputs)
-        dev_tok, tok, lp = _step(logits, temperature, top_k, _uniforms(uniform_source, step + 1, B, dev, generator), rv_dev)
+        dev_tok, tok, lp = _step(logits, temperature, top_k, _uniforms(uniform_source, step + 1, B, dev, generator), rv_dev,
+                                 active)
         ended = active & (tok == eos_token_id)                                 # node.py:369-370: EOS is not recorded
         rows = np.nonzero(active & ~ended)[0]
         toks[rows, lens[rows]] = tok[rows]                                     # node.py:371-373

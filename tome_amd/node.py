@@ -17,7 +17,7 @@ from typing import Any, Callable, List, Optional, Sequence
 import numpy as np
 import torch
 
-from .wire import pack_ref_work, scatter_ref_logprobs
+from .wire import PackedRefChunk, iter_ref_work, scatter_ref_logprobs
 from .logprob import fused_lmhead_logprobs, token_logprobs_rows
 
 logger = logging.getLogger(__name__)
@@ -72,39 +72,98 @@ class RefLogprobServicer:
         self.norm_eps = norm_eps                          # RMSNorm default, model.py:337
         self.last_ref_tokens = 0
         self.last_ref_seconds = 0.0
+        self._slots = None                                # created on first use (needs the GPU)
 
     async def _process_ref_logprobs_batched(self, prompts: Sequence, results: Sequence, G: int,
                                             temperature: float = 1.0) -> None:
         """Compute reference-model log-probs of every completion token, batched, without KV cache."""
         self.process_ref_logprobs_batched(prompts, results, G, temperature)
 
+    # ---- staging: one pinned host buffer and one device buffer per pipeline slot, grown on demand ----------
+    def _slot(self, i: int, in_bytes: int, out_floats: int) -> "_Slot":
+        if self._slots is None:
+            self._slots = [_Slot(), _Slot()]
+        slot = self._slots[i]
+        if slot.host_in is None or slot.host_in.numel() < in_bytes:
+            cap = max(in_bytes, 1 << 16) * 3 // 2
+            slot.host_in = torch.empty(cap, dtype=torch.uint8, pin_memory=True)
+            slot.dev_in = torch.empty(cap, dtype=torch.uint8, device=self.device)
+        if slot.host_out is None or slot.host_out.numel() < out_floats:
+            slot.host_out = torch.empty(max(out_floats, 1 << 12) * 3 // 2, dtype=torch.float32, pin_memory=True)
+        return slot
+
+    def _launch(self, chunk: PackedRefChunk, slot_index: int, temp: float) -> "_Slot":
+        """Everything one chunk puts on the stream: ONE upload (ids, scored rows, targets), the model's forward,
+        the log-prob kernel over the scored rows only, and the download of the packed result.  Nothing here waits
+        for the GPU."""
+        nb, max_len = chunk.ids.shape
+        n = chunk.n_scored
+        id_bytes, n_bytes = nb * max_len * 8, n * 4
+        slot = self._slot(slot_index, id_bytes + 2 * n_bytes, n)
+        host = slot.host_in.numpy()
+        host[:id_bytes].view(np.int64)[:] = chunk.ids.reshape(-1)
+        host[id_bytes:id_bytes + n_bytes].view(np.int32)[:] = chunk.scored_rows
+        host[id_bytes + n_bytes:id_bytes + 2 * n_bytes].view(np.int32)[:] = chunk.scored_targets
+        total = id_bytes + 2 * n_bytes
+        slot.dev_in[:total].copy_(slot.host_in[:total], non_blocking=True)
+        full_ids = slot.dev_in[:id_bytes].view(torch.int64).view(nb, max_len)
+        rows = slot.dev_in[id_bytes:id_bytes + n_bytes].view(torch.int32)
+        tg = slot.dev_in[id_bytes + n_bytes:total].view(torch.int32)
+        out, _ = self.reference_model(full_ids, cache=None)               # node.py:443
+        # The scored positions - rows p_len-1 .. p_len-2+len(c) of each sequence (node.py:449) - in row-major order.
+        if self.lm_head_weight is None:
+            lps = token_logprobs_rows(out, rows, tg, temp).lp             # only the listed rows are launched
+        else:
+            picked = out.reshape(nb * max_len, out.shape[-1]).index_select(0, rows.long())   # completion rows only
+            lps = fused_lmhead_logprobs(picked, self.lm_head_weight, tg, temp,
+                                        norm_weight=self.final_norm_weight, norm_eps=self.norm_eps).lp
+        slot.host_out[:n].copy_(lps, non_blocking=True)                   # node.py:456: the one copy back, of n floats
+        slot.done.record(torch.cuda.current_stream(self.device))
+        slot.chunk, slot.keep = chunk, (out, lps)                         # outputs stay alive until they have been read
+        return slot
+
+    def _finish(self, slot: "_Slot", results: Sequence) -> int:
+        slot.done.synchronize()
+        n = slot.chunk.n_scored
+        written = scatter_ref_logprobs(slot.chunk, slot.host_out.numpy()[:n], results)   # node.py:457-458
+        slot.chunk = slot.keep = None
+        return written
+
     def process_ref_logprobs_batched(self, prompts: Sequence, results: Sequence, G: int,
                                      temperature: float = 1.0) -> None:
-        """Synchronous body of ``_process_ref_logprobs_batched`` (the reference's coroutine has no awaits)."""
+        """Synchronous body of ``_process_ref_logprobs_batched`` (the reference's coroutine has no awaits).
+
+        Chunks run one deep in a pipeline: chunk i + 1 is packed on the host and put on the stream before the
+        result of chunk i is waited for, so host bookkeeping and GPU work overlap.  Results are appended in chunk
+        order, as the reference does.  (Two chunks' model outputs are alive at a time.)"""
         t0 = time.perf_counter()
         num_toks = 0
         temp = temperature or 1.0                                         # node.py:451
+        pending = None
+        turn = 0
         # work list, chunks of max_ref_batch_size, right-padding with id 0: node.py:409-441
-        for chunk in pack_ref_work(prompts, results, G, self.max_ref_batch_size):
+        for chunk in iter_ref_work(prompts, results, G, self.max_ref_batch_size):
             if chunk.n_scored == 0:                                      # only empty completions (node.py:428-432)
                 continue
-            full_ids = torch.from_numpy(chunk.ids).to(self.device)
-            out, _ = self.reference_model(full_ids, cache=None)           # node.py:443
-            # The scored positions - rows p_len-1 .. p_len-2+len(c) of each sequence (node.py:449) - packed in
-            # row-major order; one sync + one copy per chunk (node.py:456), of those positions only.
-            if self.lm_head_weight is None:
-                rows = torch.from_numpy(chunk.scored_rows).to(self.device)
-                tg = torch.from_numpy(chunk.scored_targets).to(self.device)
-                flat = token_logprobs_rows(out, rows, tg, temp).lp.cpu().numpy()   # only the listed rows are launched
-            else:
-                tg = torch.from_numpy(chunk.targets).to(self.device)
-                rv = torch.from_numpy(chunk.valid).to(self.device)
-                lps = fused_lmhead_logprobs(out, self.lm_head_weight, tg, temp, row_valid=rv,
-                                            norm_weight=self.final_norm_weight, norm_eps=self.norm_eps).lp
-                flat = lps[rv.bool()].cpu().numpy()
-            num_toks += scatter_ref_logprobs(chunk, flat, results)        # node.py:457-458
+            with torch.cuda.device(self.device):
+                slot = self._launch(chunk, turn & 1, temp)
+            turn += 1
+            if pending is not None:
+                num_toks += self._finish(pending, results)
+            pending = slot
+        if pending is not None:
+            num_toks += self._finish(pending, results)
 
         elapsed = time.perf_counter() - t0
         self.last_ref_tokens, self.last_ref_seconds = num_toks, elapsed
         logger.info("Ref log-probs non-KV batched completed: %d tokens in %.2fs (%.1f tok/s)",
                     num_toks, elapsed, num_toks / elapsed if elapsed > 0 else 0.0)
+
+
+class _Slot:
+    """Staging buffers and the completion event of one chunk in flight."""
+
+    def __init__(self):
+        self.host_in = self.dev_in = self.host_out = None
+        self.done = torch.cuda.Event()
+        self.chunk = self.keep = None
