@@ -552,7 +552,7 @@ def bench_full_matrix(dev, steps, warmup, rows, dtype_name):
     torch.cuda.synchronize()
     sample = torch.arange(0, rows, max(1, rows // 16), device=dev)[:16]     # gate: 16 rows against torch in fp64
     want = torch.log_softmax(xs[0][sample].double(), dim=-1)
-    tol = 1e-4 if dtype_name == "f32" else 0.0625 + 1e-6                     # bf16 output: one ulp at |x| < 16
+    tol = 1e-4 if dtype_name == "f32" else 0.25                              # bf16 output and subtraction: two ulps at |x| in [16, 32)
     assert (outs[0][sample].double() - want).abs().max().item() <= tol
     tm = time_steps(step, steps, warmup)
     tm.update({"rows": rows, "bytes": 3 * rows * V * esize})

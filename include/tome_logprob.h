@@ -160,15 +160,16 @@ int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows
  * Needs H % 8 == 0 and 16-byte aligned rows; row strides below 2^31 elements.  With H % 64 != 0
  * (the generic kernel, 32-bit byte offsets) hidden and weight must each span less than 4 GiB.
  *
- * Process-wide state of the library, all of it caches that do not change results: the CU count
- * of the first GPU used (one workgroup per CU for batches of up to 128 tokens), a flag per large-LDS
- * kernel ("dynamic LDS limit raised"), the device address of tome_row_logprob_noalloc's array,
- * and the selector below.
+ * Process-wide state of the library, all of it caches that do not change results and all of it kept per
+ * device ordinal: the CU count (one workgroup per CU for batches of up to 128 tokens), a flag per large-LDS
+ * kernel ("dynamic LDS limit raised"), the device address of tome_row_logprob_noalloc's array; and the
+ * two testing hooks (the selector below, tome_row_logprob_noalloc_limit).
  */
 /* Testing and tuning hook, no counterpart in the reference: kind 0 / 1 makes the fused entry points take
- * the generic / LDS-DMA sweep kernel wherever its shape rules allow, 3 / 4 the LDS-DMA kernel with
- * 256-row / 224-row vocab tiles, -1 (the default, also for any other value) picks by shape.
- * Process-wide; set it while no call of this library is running. */
+ * the generic / LDS-DMA sweep kernel wherever its shape rules allow, 3 the LDS-DMA kernel with every vocab
+ * range cut at whole 256-row tiles (no 224-row tiles, no mixed tile heights), -1 (the default, also for any
+ * other value) picks by shape.  Process-wide; set it while no call of this library is running; not for
+ * production callers. */
 void tome_select_fused_kernel(int kind);
 size_t tome_fused_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V);
 int tome_fused_lmhead_logprob(const void* hidden, const void* weight, int64_t n_tokens, int64_t H,

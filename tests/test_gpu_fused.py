@@ -17,10 +17,10 @@ TOL = 2e-3
 
 @pytest.fixture
 def force_kernel():
-    """tome_select_fused_kernel for one test: 'generic' / 'dma' force that sweep kernel, 'dma256' / 'dma224' the
-    LDS-DMA kernel with that vocab-tile height; reset afterwards."""
+    """tome_select_fused_kernel for one test: 'generic' / 'dma' force that sweep kernel, 'dma_whole_tiles' the LDS-DMA
+    kernel with vocab ranges cut at whole 256-row tiles (no short last tile); reset afterwards."""
     lib = tome_amd.load_library()
-    yield lambda kind: lib.tome_select_fused_kernel({"generic": 0, "dma": 1, "dma256": 3, "dma224": 4}[kind])
+    yield lambda kind: lib.tome_select_fused_kernel({"generic": 0, "dma": 1, "dma_whole_tiles": 3}[kind])
     lib.tome_select_fused_kernel(-1)
 
 
@@ -183,7 +183,7 @@ def test_fused_argmax_spike_and_ties(dev):
     assert (masked.argmax.cpu().numpy() == -1).all()
 
 
-@pytest.mark.parametrize("kind", ["generic", "dma", "dma256", "dma224"])
+@pytest.mark.parametrize("kind", ["generic", "dma", "dma_whole_tiles"])
 def test_fused_every_kernel_path(dev, kind, force_kernel):
     """The two GEMM kernels behind tome_fused_lmhead_logprob (generic / LDS-DMA) are picked
     by shape; tome_select_fused_kernel forces each of them onto the same problem."""
@@ -202,18 +202,45 @@ def test_fused_every_kernel_path(dev, kind, force_kernel):
     assert (r.lp.cpu().numpy()[~m] == 0).all() and (r.argmax.cpu().numpy()[~m] == -1).all()
 
 
-@pytest.mark.parametrize("n,H,V", [(50, 128, 224 * 3), (100, 192, 224 * 5 + 7), (256, 1024, 20000), (200, 64, 223), (1000, 256, 4481)])
+def _dma_tail_heights(n, V):
+    """The short-tile heights (16-row blocks per wave, 0 = none) the LDS-DMA kernel meets on this shape: a host-side
+    restatement of how it deals the vocab axis - 32-row units, `splits` contiguous ranges, whole 256-row tiles first.
+    Valid where all workgroups run in one round (token tiles * 8 <= 256), which is every shape this is used on."""
+    bt = 256 if n > 128 else (128 if n > 64 else 64)
+    tt = -(-n // bt)
+    assert tt * 8 <= 256
+    units, tiles = -(-V // 32), -(-V // 256)
+    splits = max(1, min(256 // tt, tiles))
+    return {((s + 1) * units // splits - s * units // splits) % 8 for s in range(splits)}
+
+
+# vocabulary sizes whose ranges end in short tiles of every height, for 256-, 128- and 64-token tiles (n > 128, > 64, <= 64):
+# with fewer splits than tiles a range is (units / splits) 32-row units long, i.e. a tail of that modulo 8
+TAIL_SHAPES = [(1000, 64, 18432), (1000, 128, 21504), (600, 64, 33920), (1000, 64, 28992), (100, 64, 77824), (100, 128, 93312),
+               (50, 64, 108096), (50, 192, 32 * (256 * 9 + 10) + 5), (256, 1024, 20000), (200, 64, 223), (1000, 256, 4481)]
+
+
+def test_tail_shapes_cover_every_short_tile_height():
+    seen = {256: set(), 128: set(), 64: set()}
+    for n, _, V in TAIL_SHAPES:
+        seen[256 if n > 128 else (128 if n > 64 else 64)] |= _dma_tail_heights(n, V)
+    assert seen[256] >= set(range(8)) and seen[128] >= {1, 2, 3, 4} and seen[64] >= {1, 2, 5, 6}
+
+
+@pytest.mark.parametrize("n,H,V", TAIL_SHAPES)
 def test_fused_tile_heights_agree(dev, n, H, V, force_kernel):
-    """The LDS-DMA kernel with 256-row and with 224-row vocab tiles (64-, 128- and 256-token tiles): each against the
-    oracle, targets placed on the first and last rows of 224-row and 256-row tiles, and the argmax of both equal."""
+    """The LDS-DMA kernel deals the vocab axis in 32-row units: a workgroup's range is whole 256-row tiles plus at most
+    one short tile of 1 .. 7 sixteen-row blocks per wave.  Every height (the shapes above cover 0 .. 7 on 64-, 128- and
+    256-token tiles) against the oracle, targets on the first and last rows of tiles, units and blocks; and the same
+    problem with ranges of whole tiles only must name the same argmax."""
     h, w, t = _inputs(dev, n, H, V, seed=n + V, w_scale=0.1)
-    edges = [v for v in (0, 111, 112, 223, 224, 255, 256, 447, 448, V - 1) if v < V]
-    t[: len(edges)] = edges
+    edges = [v for v in (0, 15, 16, 31, 32, 111, 112, 127, 128, 223, 224, 255, 256, 447, 448, V - 33, V - 32, V - 1) if 0 <= v < V]
+    t[: len(edges)] = edges[: n]
     valid = np.ones(n, dtype=np.int32)
     valid[n // 3] = 0
     want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(w), t, 0.9)
     got = {}
-    for kind in ("dma256", "dma224"):
+    for kind in ("dma", "dma_whole_tiles"):
         force_kernel(kind)
         r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 0.9, want_lse=True, want_entropy=True,
                                            want_argmax=True, row_valid=torch.from_numpy(valid).to(dev))
@@ -224,10 +251,10 @@ def test_fused_tile_heights_agree(dev, n, H, V, force_kernel):
         check_argmax(h, w, r.argmax.cpu().numpy(), want, 0.9, rows=np.flatnonzero(m), min_clear=0.0)
         assert r.lp.cpu().numpy()[n // 3] == 0 and r.argmax.cpu().numpy()[n // 3] == -1
         got[kind] = r.argmax.cpu().numpy()
-    np.testing.assert_array_equal(got["dma256"], got["dma224"])
+    np.testing.assert_array_equal(got["dma"], got["dma_whole_tiles"])
 
 
-@pytest.mark.parametrize("kind", ["generic", "dma", "dma224"])
+@pytest.mark.parametrize("kind", ["generic", "dma", "dma_whole_tiles"])
 @pytest.mark.parametrize("n,frac_valid", [(300, 1.0), (2304, 1.0), (9000, 1.0), (9000, 0.45), (20000, 0.8)])
 def test_fused_every_partial_is_written(dev, kind, n, frac_valid, force_kernel):
     """The work decomposition (token tiles x vocab splits, one or several rounds of workgroups, chosen on

@@ -5,7 +5,22 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace tome {
+
+// Host-side "done once per GPU" flag for settings that the runtime keeps per device (hipFuncSetAttribute): a bit per
+// device ordinal.  Losing a race repeats the setting, which is harmless.
+constexpr int kMaxDeviceOrdinals = 64;
+struct DeviceOnce {
+  std::atomic<uint64_t> done{0};
+  bool first_on_current_device() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDeviceOrdinals) return true;  // cannot tell: set again
+    const uint64_t bit = 1ull << dev;
+    return (done.fetch_or(bit, std::memory_order_relaxed) & bit) == 0;
+  }
+};
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;

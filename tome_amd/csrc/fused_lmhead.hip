@@ -68,11 +68,13 @@ struct FusedPartial {  // 32 bytes per (token, part)
 struct FusedSchedule {
   int n_ttiles, n_splits, n_wg, pad;
 };
-__host__ __device__ inline int64_t fused_split_cost(int n_ttiles, int n_splits, int slots, int n_vtiles) {
+// The vocab axis is dealt to the splits in UNITS: whole 256-row tiles for the generic kernel (one unit per tile), 32-row
+// units for the DMA kernel (eight per tile), whose last tile of a range may be shorter than 256 rows.  `upt` = units per tile.
+__host__ __device__ inline int64_t fused_split_cost(int n_ttiles, int n_splits, int slots, int n_vunits, int upt) {
   const int rounds = (n_ttiles * n_splits + slots - 1) / slots;
-  const int longest = (n_vtiles + n_splits - 1) / n_splits;
+  const int longest = (n_vunits + n_splits - 1) / n_splits;  // in units
   const int pen64 = 60 + 32 / (n_splits < 8 ? n_splits : 8);
-  return ((int64_t)rounds * (2 * longest + 1) * pen64) * 64 + n_splits;  // ties go to fewer splits
+  return ((int64_t)rounds * (2 * longest + upt) * pen64) * 64 + n_splits;  // ties go to fewer splits
 }
 __host__ __device__ inline int fused_ttiles(int n_valid, int bt) {
   const int t = (n_valid + bt - 1) / bt;
@@ -80,12 +82,13 @@ __host__ __device__ inline int fused_ttiles(int n_valid, int bt) {
 }
 __host__ __device__ inline int fused_one_round_splits(int n_ttiles, int slots, int n_vtiles) {
   int sp = slots / n_ttiles;
-  if (sp > n_vtiles) sp = n_vtiles;
+  if (sp > n_vtiles) sp = n_vtiles;  // every split keeps at least one tile's worth of rows
   return sp < 1 ? 1 : sp;
 }
 constexpr int kSplitCandidates = 32;
-inline FusedSchedule fused_schedule(int n_valid, int bt, int slots, int n_vtiles) {  // host
+inline FusedSchedule fused_schedule(int n_valid, int bt, int slots, int n_vunits, int upt) {  // host
   FusedSchedule s;
+  const int n_vtiles = (n_vunits + upt - 1) / upt;
   s.n_ttiles = fused_ttiles(n_valid, bt);
   s.pad = 0;
   if (s.n_ttiles * 8 <= slots) {
@@ -93,7 +96,7 @@ inline FusedSchedule fused_schedule(int n_valid, int bt, int slots, int n_vtiles
   } else {
     int64_t best = INT64_MAX;
     for (int c = 1; c <= kSplitCandidates && c <= n_vtiles; ++c) {
-      const int64_t cost = fused_split_cost(s.n_ttiles, c, slots, n_vtiles);
+      const int64_t cost = fused_split_cost(s.n_ttiles, c, slots, n_vunits, upt);
       if (cost < best) best = cost;
     }
     s.n_splits = (int)(best & 63);
@@ -102,15 +105,16 @@ inline FusedSchedule fused_schedule(int n_valid, int bt, int slots, int n_vtiles
   return s;
 }
 // The same on the device, by one whole wave: lane c prices c + 1 splits.
-__device__ inline FusedSchedule fused_schedule_wave(int n_valid, int bt, int slots, int n_vtiles, int lane) {
+__device__ inline FusedSchedule fused_schedule_wave(int n_valid, int bt, int slots, int n_vunits, int upt, int lane) {
   FusedSchedule s;
+  const int n_vtiles = (n_vunits + upt - 1) / upt;
   s.n_ttiles = fused_ttiles(n_valid, bt);
   s.pad = 0;
   if (s.n_ttiles * 8 <= slots) {
     s.n_splits = fused_one_round_splits(s.n_ttiles, slots, n_vtiles);
   } else {
     const int c = lane + 1;
-    int64_t cost = (c <= kSplitCandidates && c <= n_vtiles) ? fused_split_cost(s.n_ttiles, c, slots, n_vtiles) : INT64_MAX;
+    int64_t cost = (c <= kSplitCandidates && c <= n_vtiles) ? fused_split_cost(s.n_ttiles, c, slots, n_vunits, upt) : INT64_MAX;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
       const int64_t o = __shfl_xor(cost, off, 64);
@@ -157,10 +161,11 @@ struct FusedArgs {
   uint32_t hidden_stride_b;  // bytes
   uint32_t weight_stride_b;
   uint32_t hidden_bytes;     // extent of the hidden matrix (< 4 GiB, checked on the host)
+  int unit32;                // DMA kernel: 32-row blocks per vocab unit (1, or 7 / 8 when ranges are whole tiles of 224 / 256 rows)
   int n_tokens;
   int H;
   int V;
-  int n_vtiles;
+  int n_vunits;              // vocab units the splits share out: 256-row tiles (generic kernel) or 32-row units (DMA kernel)
   int slots;                 // workgroups that fit the chip at once (the schedule aims at one round)
   float scale;               // log2(e) / temperature
   FusedSchedule sched;       // host-computed schedule (no mask)
@@ -290,8 +295,8 @@ __global__ __launch_bounds__(kFusedWG, 2) void fused_lmhead_kernel(FusedArgs a) 
   int ttile, split;
   if (n_valid <= 0 || !fused_locate(sch, blockIdx.x, ttile, split)) return;
   const int t0 = ttile * kBT;
-  const int vt0 = (int)((int64_t)split * a.n_vtiles / sch.n_splits);
-  const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / sch.n_splits);
+  const int vt0 = (int)((int64_t)split * a.n_vunits / sch.n_splits);  // one unit = one 256-row tile here
+  const int vt1 = (int)((int64_t)(split + 1) * a.n_vunits / sch.n_splits);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wave_v = wave & 1, wave_t = wave >> 1;
@@ -402,8 +407,9 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 // Fold one wave tile (NBV x NBT blocks of 16x16) into the per-token running states.  Element e of
 // block i holds vocab row  vw0 + i*16 + 4*g + e  (g = lane / 16) for the token of block column j.
-template <bool ENT, bool AMAX, int NBV, int NBT>
-__device__ __forceinline__ void fold_tile16(f32x4v (&acc)[NBV][NBT], RowStat (&st)[NBT], float (&tx)[NBT],
+// NBV of the NBV_ALLOC block rows the array holds are folded (a short tile uses the first few).
+template <bool ENT, bool AMAX, int NBV, int NBT, int NBV_ALLOC>
+__device__ __forceinline__ void fold_tile16(f32x4v (&acc)[NBV_ALLOC][NBT], RowStat (&st)[NBT], float (&tx)[NBT],
                                             const int (&tgt)[NBT], int vw0, int g, bool partial_tile, int V,
                                             float scale) {
   if (partial_tile) {  // last vocab tile: rows past V do not exist
@@ -572,17 +578,25 @@ __device__ __forceinline__ void pair_reads() {
   }
 }
 
-// HI: vocab blocks in the second half of a wave's tile, 4 or 3.  With 3 the workgroup tile is 224 vocab rows (2 x 7 blocks)
-// instead of 256: the schedule takes it where whole 256-row tiles would leave the workgroups of a launch that streams W
-// once with uneven shares (594 tiles over 256 workgroups: three for some, two for the others).  The slab keeps its 256
-// rows in LDS; the 32 unused ones are requested as copies of rows the same instruction fetches anyway.
+// Vocab ranges are dealt in units of 32 rows and a workgroup cuts its range into the fewest tiles of at most 256 rows,
+// all of the same height or one unit apart (the taller ones first): V = 151936 over 16 splits is 297 units per
+// workgroup = 31 tiles of 256 rows + 7 of 224, where whole 256-row tiles would give some workgroups 38 tiles and others
+// 37 - and a tile costs its full MFMA work however few of its rows count.  A tile of nb blocks of 16 rows per wave
+// (nb = 1 .. 8) runs the same pipeline with 8 * nb MFMAs per wave and step.  Its slab keeps the LDS layout of a whole
+// tile (rows 0..127 for the waves of vocab half 0, 128..255 for half 1, so fragment addresses do not change); each
+// half holds 16 * nb rows of W and the rest of its LDS rows are requested as copies of its last row and never multiplied.
 template <bool ENT, bool AMAX, int NBT, int HI>
 __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  static_assert(HI == 4 || HI == 3, "tile heights: 256 or 224 vocab rows");
-  constexpr int kNBVw = 4 + HI;                     // 16-row vocab blocks per wave
-  constexpr int kWaveRows = kNBVw * 16;             // vocab rows per wave
-  constexpr int kTileRows = 2 * kWaveRows;          // vocab rows per workgroup tile
+  static_assert((NBT == 4 && (HI == 4 || HI == 3)) || (NBT != 4 && HI == 0), "256-token tile: every vocab tile 256 (HI = 4) or 224 rows; others: mixed heights");
+  // The 256-token tile runs at the limit of the register file: it keeps ONE tile height per launch (4 + HI blocks per wave,
+  // the host picks 256 or 224 rows), because the code for two or more heights in one kernel costs it 60 and more spilled
+  // registers whose reloads, at every tile change, wait for memory behind the W stream (measured with heights of 224 and
+  // 256 rows mixed: +8 % at 4096 x 1024 instead of the 1.7 % that the even shares would save).  The smaller token tiles
+  // have registers to spare and mix heights as described above.
+  constexpr bool kMixed = HI == 0;
+  constexpr int kMaxBlocks = kMixed ? 8 : 4 + HI;   // 16-row vocab blocks per wave in the tallest tile
+  constexpr int kNBVw = 8;                          // accumulator block rows per wave
   constexpr int k2NBT = NBT;                        // 16-token blocks per wave
   constexpr int k2BT = dma_tile_tokens(NBT);        // tokens per workgroup
   constexpr int kWaveTok = NBT * 16;                // tokens per wave
@@ -608,8 +622,22 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   int ttile, split;
   if (n_valid <= 0 || !fused_locate(sch, blockIdx.x, ttile, split)) return;
   const int t0 = ttile * k2BT;
-  const int vt0 = (int)((int64_t)split * a.n_vtiles / sch.n_splits);
-  const int vt1 = (int)((int64_t)(split + 1) * a.n_vtiles / sch.n_splits);
+  // This workgroup's vocab range in 32-row blocks (a.unit32 = blocks per unit: 1, or 7 / 8 when ranges are whole tiles).
+  const int u0 = (int)((int64_t)split * a.n_vunits / sch.n_splits) * a.unit32;
+  const int u1 = (int)((int64_t)(split + 1) * a.n_vunits / sch.n_splits) * a.unit32;
+  const int n_units = u1 - u0;                      // >= 1: every split holds at least one unit
+  // With mixed heights every workgroup of a launch cuts its range into the SAME number of tiles (the longest range's), so
+  // that all of them step through tiles of (nearly) the same heights at the same time: the workgroups that share a
+  // hidden-state or W stream in an XCD's L2 only hit there while they stay in step.
+  const int n_tiles = kMixed ? ((a.n_vunits + sch.n_splits - 1) / sch.n_splits * a.unit32 + 7) >> 3 : n_units / kMaxBlocks;
+  const int nb_short = kMixed ? n_units / n_tiles : kMaxBlocks;  // 16-row blocks per wave of the shorter tiles (1 .. 8)
+  const int n_tall = kMixed ? n_units - nb_short * n_tiles : 0;  // tiles with one block more: they come first
+  const int row0 = u0 * 32;
+  auto tile_blocks = [&](int tile) { return nb_short + (tile < n_tall ? 1 : 0); };
+  auto tile_row0 = [&](int tile) {
+    if constexpr (!kMixed) return row0 + tile * (32 * kMaxBlocks);
+    else return row0 + 32 * (tile * nb_short + (tile < n_tall ? tile : n_tall));
+  };
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps LDS bases scalar
@@ -623,19 +651,35 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   const int dc = (lane & 7) ^ (4 * (wave & 1) + (dr >> 1));   // global chunk: position ^ ((row >> 1) & 7)
   const char* pa[k2Loads];  // next W slab to request, per DMA instruction
   const char* pb[kBLoads];  // next hidden slab
-  auto point_a = [&](int vt) {  // rows past V (last tile only) read the last row; masked in the epilogue
+  // Mixed heights: LDS row r of a W slab holds vocab row  base + (r / 128) * wr + min(r % 128, wr - 1)  of tile `tile`,
+  // wr = rows per wave of that tile.  One height: LDS row r is tile row r; the 32 LDS rows past a 224-row tile are requested
+  // as copies of rows that waves 0-3 fetch with the same instruction.  Rows past V (last tile only) read the last row
+  // and are masked in the epilogue.
+  auto point_a = [&](int tile) {
+    const int64_t base = tile_row0(tile);
+    const int wr = kMixed ? tile_blocks(tile) * 16 : kMaxBlocks * 16;
+    // The lane's row and chunk are derived afresh here (the empty asm hides that they are loop invariants): hoisted
+    // out of the sweep, the 64-bit per-lane address terms built from them would stay live across every step, and this
+    // kernel has no register left for them.
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int dr = ln >> 3;
+    const int dc = (ln & 7) ^ (4 * (wave & 1) + (dr >> 1));
 #pragma unroll
     for (int j = 0; j < k2Loads; ++j) {
-      int64_t v = (int64_t)vt * kTileRows + (j * 8 + wave) * 8 + dr;  // tile row = LDS row of the slab
-      if constexpr (HI != 4) {  // LDS rows past the tile: a copy of what waves 0-3 request with this instruction
-        const int r = (j * 8 + wave) * 8 + dr;
-        v = (int64_t)vt * kTileRows + (r < kTileRows ? r : r - 32);
+      const int r = (j * 8 + wave) * 8 + dr;
+      int64_t v;
+      if constexpr (kMixed) {
+        const int in_half = (r & 127) < wr ? (r & 127) : wr - 1;
+        v = base + (r >> 7) * wr + in_half;
+      } else {
+        v = base + ((HI == 4 || r < 2 * wr) ? r : r - 32);
       }
       v = v < a.V ? v : a.V - 1;
       pa[j] = a.weight + v * a.weight_stride_b + dc * 16;
     }
   };
-  point_a(vt0);
+  point_a(0);
 #pragma unroll
   for (int j = 0; j < kBLoads; ++j) {
     int p = t0 + (j * 8 + wave) * 8 + dr;
@@ -660,13 +704,14 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 
   // ---- fragment read offsets inside a slab (swizzled): lane group g reads chunk 4*ks + g ----------
   const int swz = (g ^ ((l16 >> 1) & 7)) * 16;  // sub-step k0; k1 is this ^ 64
-  const int rdA = (wave_v * kWaveRows + l16) * k2RowBytes + swz;  // kWaveRows is a multiple of 16: the swizzle term stays l16's
+  // the wave's first LDS row (128 with mixed heights) is a multiple of 16: the swizzle term stays l16's
+  const int rdA = (wave_v * (kMixed ? 128 : kMaxBlocks * 16) + l16) * k2RowBytes + swz;
   const int rdB = (wave_t * kWaveTok + l16) * k2RowBytes + swz;
 
   const int nk = a.H / k2BK;
-  const int n_steps = (vt1 - vt0) * nk;
+  const int n_steps = n_tiles * nk;
   const int64_t slab_rewind = (int64_t)(nk - 1) * k2RowBytes;
-  int i_kt = 0, i_vt = vt0;  // slab the next request fetches
+  int i_kt = 0, i_tile = 0;  // slab the next request fetches
   int issued = 0;            // slabs requested so far; request q lands in buffers q % kBufs
 
   // One of the DMA instructions of the next request (0-3: W rows; the others: hidden rows).  Past the last slab
@@ -687,10 +732,10 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
       for (int j = 0; j < kBLoads; ++j) pb[j] += k2RowBytes;
     } else {
       i_kt = 0;
-      ++i_vt;
+      ++i_tile;
 #pragma unroll
       for (int j = 0; j < kBLoads; ++j) pb[j] -= slab_rewind;
-      if (i_vt < vt1) point_a(i_vt);
+      if (i_tile < n_tiles) point_a(i_tile);
     }
   };
   // Fragments of one K = 32 sub-step of a slab: W blocks [i0, i0 + n) or the hidden blocks.
@@ -700,8 +745,6 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     for (int i = 0; i < decltype(n)::value; ++i)
       fa[i] = *reinterpret_cast<const bf16x8*>(slab + (rdA ^ (ks * 64)) + (i0 + i) * 16 * k2RowBytes);
   };
-  constexpr std::integral_constant<int, 4> kLo{};
-  constexpr std::integral_constant<int, HI> kHi{};
   auto read_b = [&](int slot, int ks, bf16x8 (&fb)[k2NBT]) {
     const char* slab = smem + kHBase + ((unsigned)slot % kBufs) * kHBytes;
 #pragma unroll
@@ -723,8 +766,9 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kInFlightAtStart) : "memory");
   __builtin_amdgcn_s_barrier();
 
+  constexpr std::integral_constant<int, 4> kFour{};
   bf16x8 fa_lo[4], fa_hi[4], fb0[k2NBT], fb1[k2NBT];
-  read_a(0, 0, 0, fa_lo, kLo);
+  read_a(0, 0, 0, fa_lo, kFour);
   read_b(0, 0, fb0);
 
   f32x4v acc[kNBVw][k2NBT];
@@ -735,7 +779,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
-  // 16 (12) MFMAs on four (three) vocab blocks; the group barriers then put one LDS read or DMA request behind
+  // 4 * n MFMAs on n vocab blocks; in a whole tile the group barriers then put one LDS read or DMA request behind
   // every MFMA (or every second one), so that its issue hides under the MFMA's execution.
   // `fresh`: the first K sub-step of a vocab tile starts from a zero C operand, which saves clearing
   // the 128 accumulator registers after every fold.
@@ -757,24 +801,28 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
       __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM (DMA request)
     }
   };
-  auto do_step = [&](auto fresh) {
+  // One K slab on a tile of `lo` + `hi` vocab blocks per wave: lo = min(nb, 4), hi = nb - lo.  The fragments of the
+  // NEXT step's first quarter are always read for four blocks (the next step may belong to a taller tile).
+  auto do_step = [&](auto fresh, auto lo, auto hi) {
+    constexpr int LO = decltype(lo)::value, HIB = decltype(hi)::value;
+    constexpr bool kTuned = NBT == 4 && LO == 4 && HIB >= 3;  // the interleave below is written for tiles of 224 and 256 rows
     __builtin_amdgcn_sched_barrier(0);
-    read_a(step, 0, 4, fa_hi, kHi);
+    read_a(step, 0, 4, fa_hi, hi);
 #pragma unroll
     for (int piece = kP4; piece < kP4 + kP1; ++piece) issue_piece(piece);  // second portion of the request for slab step + 1
-    mfma_half(0, fa_lo, fb0, fresh, kLo);
-    if constexpr (NBT == 4) {
-      pair_reads<2, HI>();
+    mfma_half(0, fa_lo, fb0, fresh, lo);
+    if constexpr (kTuned) {
+      pair_reads<2, HIB>();
       pair_dma(std::integral_constant<int, kP1>{});
     }
     __builtin_amdgcn_sched_barrier(0);
-    read_a(step, 1, 0, fa_lo, kLo);
+    read_a(step, 1, 0, fa_lo, lo);
     read_b(step, 1, fb1);
 #pragma unroll
     for (int piece = kP4 + kP1; piece < k2DmaPerSlab; ++piece) issue_piece(piece);  // third portion
-    mfma_half(4, fa_hi, fb0, fresh, kHi);
-    if constexpr (NBT == 4) {
-      if constexpr (kP2 == 0 && HI == 4) {
+    mfma_half(4, fa_hi, fb0, fresh, hi);
+    if constexpr (kTuned) {
+      if constexpr (kP2 == 0) {
         pair_reads<2, 8>();
       } else {
         pair_reads<1, 8>();
@@ -783,9 +831,9 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (kP4 < k2DmaPerSlab) issue_done();
-    read_a(step, 1, 4, fa_hi, kHi);
-    mfma_half(0, fa_lo, fb1, std::false_type{}, kLo);
-    if constexpr (NBT == 4) pair_reads<2, HI>();
+    read_a(step, 1, 4, fa_hi, hi);
+    mfma_half(0, fa_lo, fb1, std::false_type{}, lo);
+    if constexpr (kTuned) pair_reads<2, HIB>();
     __builtin_amdgcn_sched_barrier(0);
     // This wave has read all it needs of slab `step` and its share of slab step+1 has landed; after
     // the (fence-less) barrier both hold for everyone.  (With three buffers the request of slab step+2
@@ -796,12 +844,12 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     // first portion of the next request, which refills the buffers of slab `step`.  The DMA requests write
     // LDS, so they keep their program order after the fragment reads.
     __builtin_amdgcn_sched_barrier(0);
-    read_a(step + 1, 0, 0, fa_lo, kLo);
+    read_a(step + 1, 0, 0, fa_lo, kFour);
     read_b(step + 1, 0, fb0);
 #pragma unroll
     for (int piece = 0; piece < kP4; ++piece) issue_piece(piece);
-    mfma_half(4, fa_hi, fb1, std::false_type{}, kHi);
-    if constexpr (NBT == 4) {
+    mfma_half(4, fa_hi, fb1, std::false_type{}, hi);
+    if constexpr (kTuned) {
       pair_reads<1, 8>();
       pair_dma(std::integral_constant<int, kP4>{});
     }
@@ -810,11 +858,41 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     ++step;
   };
 
-  for (int vt = vt0; vt < vt1; ++vt) {
-    do_step(std::true_type{});
-    for (int kt = 1; kt < nk; ++kt) do_step(std::false_type{});
-    const int v0 = vt * kTileRows;
-    fold_tile16<ENT, AMAX>(acc, st, tx, tgt, v0 + wave_v * kWaveRows, g, v0 + kTileRows > a.V, a.V, a.scale);
+  // Two runs of tiles: n_tall tiles of nb_short + 1 blocks, then the others of nb_short blocks.
+  auto run_tiles = [&](int first, int last, auto lo, auto hi) {
+    constexpr int NB = decltype(lo)::value + decltype(hi)::value;
+    for (int tile = first; tile < last; ++tile) {
+      do_step(std::true_type{}, lo, hi);
+      for (int kt = 1; kt < nk; ++kt) do_step(std::false_type{}, lo, hi);
+      const int v0 = tile_row0(tile);
+      fold_tile16<ENT, AMAX, NB>(acc, st, tx, tgt, v0 + wave_v * NB * 16, g, v0 + 2 * NB * 16 > a.V, a.V, a.scale);
+    }
+  };
+  using std::integral_constant;
+  if constexpr (!kMixed) {
+    constexpr integral_constant<int, HI == 0 ? 4 : HI> kHi{};
+    for (int tile = 0; tile < n_tiles; ++tile) {
+      do_step(std::true_type{}, kFour, kHi);
+      for (int kt = 1; kt < nk; ++kt) do_step(std::false_type{}, kFour, kHi);
+      const int v0 = row0 + tile * (32 * kMaxBlocks);
+      fold_tile16<ENT, AMAX, kMaxBlocks>(acc, st, tx, tgt, v0 + wave_v * kMaxBlocks * 16, g, v0 + 32 * kMaxBlocks > a.V, a.V, a.scale);
+    }
+  } else {
+    for (int run = 0; run < 2; ++run) {
+      const int first = run == 0 ? 0 : n_tall, last = run == 0 ? n_tall : n_tiles;
+      if (first >= last) continue;
+      const int nb = nb_short + (run == 0 ? 1 : 0);
+      switch (nb) {
+        case 1: run_tiles(first, last, integral_constant<int, 1>{}, integral_constant<int, 0>{}); break;
+        case 2: run_tiles(first, last, integral_constant<int, 2>{}, integral_constant<int, 0>{}); break;
+        case 3: run_tiles(first, last, integral_constant<int, 3>{}, integral_constant<int, 0>{}); break;
+        case 4: run_tiles(first, last, integral_constant<int, 4>{}, integral_constant<int, 0>{}); break;
+        case 5: run_tiles(first, last, integral_constant<int, 4>{}, integral_constant<int, 1>{}); break;
+        case 6: run_tiles(first, last, integral_constant<int, 4>{}, integral_constant<int, 2>{}); break;
+        case 7: run_tiles(first, last, integral_constant<int, 4>{}, integral_constant<int, 3>{}); break;
+        default: run_tiles(first, last, kFour, kFour); break;
+      }
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no request may outlive the workgroup's LDS
 
@@ -948,7 +1026,7 @@ __global__ __launch_bounds__(512) void fused_lmhead_small_kernel(FusedArgs a) {
         f32x4v sum[1][1] = {{f32x4v{0.f, 0.f, 0.f, 0.f}}};
         const char* src = small_mem + (size_t)((t & (kRed - 1)) * n_waves * NBT + wave) * 1024 + lane * 16;
         for (int w = 0; w < n_waves; ++w) sum[0][0] += *reinterpret_cast<const f32x4v*>(src + (size_t)w * NBT * 1024);
-        fold_tile16<ENT, AMAX, 1, 1>(sum, st, tx, tgt, t * 16, g, t * 16 + 16 > a.V, a.V, a.scale);
+        fold_tile16<ENT, AMAX, 1>(sum, st, tx, tgt, t * 16, g, t * 16 + 16 > a.V, a.V, a.scale);
       }
       if constexpr (kRed == 1) __syncthreads();  // one buffer: the next tile's sums wait for this fold
     }
@@ -971,7 +1049,7 @@ struct CompactArgs {
   float* out4;
   int32_t* out_argmax;
   int n;
-  int bt, slots, n_vtiles;  // inputs of the schedule, which this kernel derives from n_valid
+  int bt, slots, n_vunits, upt;  // inputs of the schedule, which this kernel derives from n_valid
 };
 
 // Rows are taken in batches of up to 16384: each of the 16 waves owns a run of consecutive rows of a batch (a
@@ -1033,7 +1111,7 @@ __global__ __launch_bounds__(1024) void compact_rows_kernel(CompactArgs a) {
   }
   if (tid == 0) *a.n_valid = done;
   if (wave == 15) {  // one wave also fixes the work decomposition, which depends on the total
-    const FusedSchedule sch = fused_schedule_wave(done, a.bt, a.slots, a.n_vtiles, lane);
+    const FusedSchedule sch = fused_schedule_wave(done, a.bt, a.slots, a.n_vunits, a.upt, lane);
     if (lane == 0) *reinterpret_cast<FusedSchedule*>(a.n_valid + 4) = sch;
   }
 }
@@ -1165,7 +1243,7 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
 // with the batch.  Decode-sized batches whose hidden states fit the waves' registers take the streaming kernel.
 
 enum FusedKind { kGeneric = 0, kDma = 1, kSmall = 2 };
-constexpr int kForceDma256 = 3, kForceDma224 = 4;  // selector values: the DMA kernel with one tile height
+constexpr int kForceDmaWholeTiles = 3;  // selector value: the DMA kernel with vocab ranges cut at whole 256-row tiles
 
 // Kernel selector for tests and tuning runs: -1 (the default) picks by shape, kGeneric / kDma force that
 // sweep kernel wherever its shape rules allow.  Process-wide; set it while no call is in flight.
@@ -1175,9 +1253,10 @@ void fused_force_kernel(int kind) { g_forced_kind.store(kind, std::memory_order_
 struct FusedPlan {
   FusedKind kind;
   int dma_nbt;                               // kDma only: token blocks per wave (4, 2 or 1: 256, 128 or 64 tokens per tile)
-  int dma_hi;                                // kDma only: 4 = 256-row vocab tiles, 3 = 224-row ones
+  int unit32;                                // kDma only: 32-row blocks per vocab unit (1 = mixed tile heights; 7 / 8 = whole tiles of 224 / 256 rows)
   int small_nbt, small_ksteps, small_waves;  // kSmall only
-  int bt, bv, slots, n_vtiles;
+  int bt, slots;
+  int n_vunits, upt;   // vocab units the splits share out, and units per 256-row tile (what a unit costs, for the schedule)
   int grid;            // workgroups to launch: the most any number of valid tokens can ask for
   size_t max_records;  // partial records any number of valid tokens can produce
 };
@@ -1192,14 +1271,16 @@ static void allow_big_lds(K kernel, int bytes) {
 // The stream is bound by the 16-rows-by-64-bytes shape of an MFMA operand load, which a plain copy
 // kernel of the same shape and lifetime moves at 5.6 TB/s, and more concurrent streams lower that.
 static int small_wg_count() {
-  static int n = 0;
+  static std::atomic<int> cached[kMaxDeviceOrdinals];  // per device ordinal: GPUs of one process may differ
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDeviceOrdinals) return 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
   if (n == 0) {
-    int cus = 0, dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 2)
-      return 0;
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 2) return 0;
     if (cus > 512) cus = 512;  // the workspace holds 512 parts per token
     n = cus & ~1;              // even: the combine kernel counts parts in pairs
+    cached[dev].store(n, std::memory_order_relaxed);
   }
   return n;
 }
@@ -1233,54 +1314,61 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   p.kind = kGeneric;
   p.small_nbt = p.small_ksteps = p.small_waves = 0;
   p.dma_nbt = n_tokens > 128 ? 4 : (n_tokens > 64 ? 2 : 1);
+  p.unit32 = 8;   // 32-row blocks per vocab unit: whole 256-row tiles unless the DMA kernel is given something finer below
   if (H % k2BK == 0) p.kind = kDma;
   // The streaming kernel runs one workgroup per CU: without a CU count (no device) the tiled kernels serve.
   if (small_shape(n_tokens, H, V, p.small_nbt, p.small_ksteps, p.small_waves) && small_wg_count() >= 2) p.kind = kSmall;
-  p.dma_hi = 4;
   const int forced = g_forced_kind.load(std::memory_order_relaxed);
   if (forced == kGeneric) p.kind = kGeneric;
-  if ((forced == kDma || forced == kForceDma256 || forced == kForceDma224) && H % k2BK == 0) p.kind = kDma;
-  p.n_vtiles = 0;
+  if ((forced == kDma || forced == kForceDmaWholeTiles) && H % k2BK == 0) p.kind = kDma;
   if (p.kind == kSmall) {
     // One partial per (token, workgroup); one workgroup per CU, at most 512.
     p.bt = 128;
-    p.bv = 16;
     p.slots = 1;     // only feed the schedule that the compaction kernel writes and this path ignores
-    p.n_vtiles = 1;
+    p.n_vunits = 1;
+    p.upt = 1;
     p.grid = 0;
     p.max_records = (size_t)128 * 512;
     return p;
   }
   p.bt = p.kind == kGeneric ? kBT : dma_tile_tokens(p.dma_nbt);   // the DMA path: 256 vocab rows x 256, 128 or 64 tokens
-  p.bv = p.kind == kGeneric ? kBV : k2BV;
-  if (p.kind == kDma) {
-    // Tile height.  Where one round of workgroups streams W once, what counts is the longest vocab range in ROWS: whole
-    // 256-row tiles deal V = 151936 as three tiles to 82 workgroups and two to the others, 224-row tiles as three to 167
-    // and two to 89 - an eighth less for the longest.  The shorter tile moves 1/7 more hidden-state bytes per MAC, so it
-    // has to win by more than that is worth (8 %), and it is only considered in the one-round regime.
-    const int tt = fused_ttiles((int)n_tokens, p.bt);
-    if (forced == kForceDma224) {
-      p.dma_hi = 3;
-    } else if (forced != kForceDma256 && tt * 8 <= 256) {
-      const int sp = fused_one_round_splits(tt, 256, 1 << 30);
-      auto longest_rows = [&](int rows) {
-        const int64_t nvt = V > 0 ? (V + rows - 1) / rows : 1;
-        const int64_t s = sp < nvt ? sp : nvt;
-        return ((nvt + s - 1) / s) * rows;
-      };
-      if (longest_rows(224) * 108 < longest_rows(256) * 100) p.dma_hi = 3;
-    }
-    if (p.dma_hi == 3) p.bv = 224;
-  }
   // resident workgroups on 256 CUs: 2 per CU, or 1 for the DMA path (80-128 KB of LDS; two 64-token workgroups of 80 KB
   // per CU measured slower than one: 288 against 277 us at 64 x 4096)
   p.slots = p.kind == kGeneric ? 512 : 256;
-  p.n_vtiles = (int)((V + p.bv - 1) / p.bv);
+  // Vocab units.  Generic kernel: whole 256-row tiles.  DMA kernel with token tiles of 64 / 128: 32-row units (tile heights
+  // are mixed inside the kernel).  DMA kernel with the 256-token tile: one tile height per launch - 256 rows, or 224 where
+  // one round of workgroups streams W once and what counts is the longest vocab range in ROWS: whole 256-row tiles deal
+  // V = 151936 as three tiles to 82 workgroups and two to the others, 224-row tiles as three to 167 and two to 89, an
+  // eighth less for the longest.  The shorter tile moves 1/7 more hidden-state bytes per MAC, so it has to win by more
+  // than that is worth (8 %), and it is only considered in the one-round regime.
+  p.n_vunits = (int)((V + kBV - 1) / kBV);
+  p.upt = 1;
+  if (p.kind == kDma && forced != kForceDmaWholeTiles) {
+    if (p.dma_nbt != 4) {
+      p.unit32 = 1;
+      p.n_vunits = (int)((V + 31) / 32);
+      p.upt = 8;
+    } else {
+      const int tt = fused_ttiles((int)n_tokens, p.bt);
+      if (tt * 8 <= 256) {
+        const int sp = fused_one_round_splits(tt, 256, 1 << 30);
+        auto longest_rows = [&](int rows) {
+          const int64_t nvt = (V + rows - 1) / rows;
+          const int64_t sv = sp < nvt ? sp : nvt;
+          return ((nvt + sv - 1) / sv) * rows;
+        };
+        if (longest_rows(224) * 108 < longest_rows(256) * 100) {
+          p.unit32 = 7;
+          p.n_vunits = (int)((V + 223) / 224);
+        }
+      }
+    }
+  }
   p.grid = 0;
   p.max_records = 0;
   const int tt_max = (int)((n_tokens + p.bt - 1) / p.bt);
   for (int tt = 1; tt <= tt_max; ++tt) {  // the schedule depends on n_valid only through its tile count
-    const FusedSchedule s = fused_schedule(tt * p.bt, p.bt, p.slots, p.n_vtiles);
+    const FusedSchedule s = fused_schedule(tt * p.bt, p.bt, p.slots, p.n_vunits, p.upt);
     const int padded = 8 * ((s.n_wg + 7) / 8);  // fused_locate deals whole rows of 8 workgroup ids
     if (padded > p.grid) p.grid = padded;
     const size_t rec = (size_t)tt * p.bt * s.n_splits * kPartsPerSplit;
@@ -1309,24 +1397,18 @@ size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weigh
 
 template <bool ENT, bool AMAX, int NBT, int HI>
 static void launch_dma_nbt(const FusedArgs& a, int grid, hipStream_t stream) {
-  static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
-  if (!attr_set) {
+  static DeviceOnce attr_set;  // opt in to > 64 KB of dynamic LDS once per instantiation and device
+  if (attr_set.first_on_current_device())
     allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI>, dma_lds_bytes(NBT));
-    attr_set = true;
-  }
   hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI>), dim3((unsigned)grid), dim3(k2WG), dma_lds_bytes(NBT),
                      stream, a);
 }
-template <bool ENT, bool AMAX, int HI>
-static void launch_dma_hi(const FusedArgs& a, int nbt, int grid, hipStream_t stream) {
-  if (nbt == 4) launch_dma_nbt<ENT, AMAX, 4, HI>(a, grid, stream);
-  else if (nbt == 2) launch_dma_nbt<ENT, AMAX, 2, HI>(a, grid, stream);
-  else launch_dma_nbt<ENT, AMAX, 1, HI>(a, grid, stream);
-}
 template <bool ENT, bool AMAX>
-static void launch_dma(const FusedArgs& a, int nbt, int hi, int grid, hipStream_t stream) {
-  if (hi == 3) launch_dma_hi<ENT, AMAX, 3>(a, nbt, grid, stream);
-  else launch_dma_hi<ENT, AMAX, 4>(a, nbt, grid, stream);
+static void launch_dma(const FusedArgs& a, int nbt, int unit32, int grid, hipStream_t stream) {
+  if (nbt == 4 && unit32 == 7) launch_dma_nbt<ENT, AMAX, 4, 3>(a, grid, stream);   // 224-row tiles
+  else if (nbt == 4) launch_dma_nbt<ENT, AMAX, 4, 4>(a, grid, stream);
+  else if (nbt == 2) launch_dma_nbt<ENT, AMAX, 2, 0>(a, grid, stream);
+  else launch_dma_nbt<ENT, AMAX, 1, 0>(a, grid, stream);
 }
 
 template <bool ENT, bool AMAX, int NBT, int KSTEPS>
@@ -1336,11 +1418,9 @@ static int launch_small(const FusedArgs& a, int waves, hipStream_t stream) {
   if (n_wg > n_tiles) n_wg = n_tiles & ~1;  // no empty vocab ranges
   if (n_wg < 2) return 0;
   const size_t lds = (size_t)(NBT == 8 ? 1 : 2) * waves * NBT * 1024 + (size_t)waves * 4096;
-  static bool attr_set = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
-  if (!attr_set && lds > 65536) {
+  static DeviceOnce attr_set;  // opt in to > 64 KB of dynamic LDS once per instantiation and device
+  if (lds > 65536 && attr_set.first_on_current_device())
     allow_big_lds(&fused_lmhead_small_kernel<ENT, AMAX, NBT, KSTEPS>, 2 * 8 * 4 * 1024 + 8 * 4096);
-    attr_set = true;
-  }
   hipLaunchKernelGGL((fused_lmhead_small_kernel<ENT, AMAX, NBT, KSTEPS>), dim3((unsigned)n_wg), dim3((unsigned)waves * 64),
                      lds, stream, a);
   return n_wg;
@@ -1364,8 +1444,8 @@ static int launch_main(const FusedArgs& a, const FusedPlan& plan, bool want_argm
     return n;  // >= 2: fused_plan only picks this kernel when it can be placed
   }
   if (plan.kind == kDma) {
-    if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.dma_hi, plan.grid, stream);
-    else launch_dma<ENT, false>(a, plan.dma_nbt, plan.dma_hi, plan.grid, stream);
+    if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.unit32, plan.grid, stream);
+    else launch_dma<ENT, false>(a, plan.dma_nbt, plan.unit32, plan.grid, stream);
   } else {
     if (want_argmax) hipLaunchKernelGGL((fused_lmhead_kernel<ENT, true>), dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
     else hipLaunchKernelGGL((fused_lmhead_kernel<ENT, false>), dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
@@ -1392,7 +1472,7 @@ static hipError_t fused_launch_impl(const void* hidden, const void* hidden_ref, 
     n_valid = reinterpret_cast<int32_t*>(ws);
     row_index = reinterpret_cast<int32_t*>(ws + off_index());
     CompactArgs c{row_valid, row_index, n_valid, out_lp, out_lse, out_entropy, out_ref_lp, out_k3, out_argmax,
-                  (int)n_tokens, plan.bt, plan.slots, plan.n_vtiles};
+                  (int)n_tokens, plan.bt, plan.slots, plan.n_vunits, plan.upt};
     hipLaunchKernelGGL(compact_rows_kernel, dim3(1), dim3(1024), 0, stream, c);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -1428,11 +1508,12 @@ static hipError_t fused_launch_impl(const void* hidden, const void* hidden_ref, 
   a.n_tokens = (int)n_tokens;
   a.H = (int)H;
   a.V = (int)V;
-  a.n_vtiles = plan.n_vtiles;
+  a.n_vunits = plan.n_vunits;
+  a.unit32 = plan.unit32;
   a.slots = plan.slots;
   // Workspace header: [0] n_valid, [16..32) the schedule derived from it on the device.
   a.sched_dev = row_valid ? reinterpret_cast<const FusedSchedule*>(n_valid + 4) : nullptr;
-  a.sched = fused_schedule((int)n_tokens, plan.bt, plan.slots, plan.n_vtiles);
+  a.sched = fused_schedule((int)n_tokens, plan.bt, plan.slots, plan.n_vunits, plan.upt);
   a.scale = kLog2e / temperature;
   FusedPartial* p0 = reinterpret_cast<FusedPartial*>(ws + off_partials(n_tokens));
   FusedPartial* p1 = reinterpret_cast<FusedPartial*>(ws + off_partials(n_tokens) + partial_bytes(n_tokens, H, V));

@@ -205,12 +205,10 @@ __global__ __launch_bounds__(kProbeWG) void mfma_ceiling_kernel(const u32x4* ope
 template <bool REQ, bool FOLD, bool BAR>
 static void mfma_probe_launch_one(const void* operands, int n_workgroups, int steps, float* sink, hipStream_t stream) {
   constexpr int lds = (REQ ? 2 : 1) * kProbeSlabBytes;
-  static bool attr_set = false;  // opt in to the large dynamic LDS once per instantiation
-  if (!attr_set) {
+  static DeviceOnce attr_set;  // opt in to the large dynamic LDS once per instantiation and device
+  if (attr_set.first_on_current_device())
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&mfma_ceiling_kernel<REQ, FOLD, BAR>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    attr_set = true;
-  }
   hipLaunchKernelGGL((mfma_ceiling_kernel<REQ, FOLD, BAR>), dim3((unsigned)n_workgroups), dim3(kProbeWG), lds, stream,
                      static_cast<const u32x4*>(operands), steps, sink);
 }
