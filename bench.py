@@ -519,9 +519,9 @@ def bench_lora(dev, steps, warmup):
 
 def bench_full_matrix(dev, steps, warmup, rows, dtype_name):
     """tome_full_log_softmax, the drop-in of fused_log_softmax (mlx-impl/model.py:77-89): the whole [rows, V] matrix
-    of log-probs in the input dtype.  Algorithmic bytes 3 * V * sizeof(T) per row (one pass for the row's lse, one
-    to read and one to write the matrix).  The small shape rotates through 16 input / output pairs so that rows come
-    from HBM, not from the last-level cache."""
+    of log-probs in the input dtype.  Algorithmic bytes: 3 * V * sizeof(T) per row with two passes (one read for the row's
+    lse, one read and one write of the matrix), 2 * V * sizeof(T) where the one-pass kernel applies.  The small shape
+    rotates through 16 input / output pairs so that rows come from HBM, not from the last-level cache."""
     import torch
     import tome_amd
     from tome_amd import _lib
@@ -555,7 +555,11 @@ def bench_full_matrix(dev, steps, warmup, rows, dtype_name):
     tol = 1e-4 if dtype_name == "f32" else 0.25                              # bf16 output and subtraction: two ulps at |x| in [16, 32)
     assert (outs[0][sample].double() - want).abs().max().item() <= tol
     tm = time_steps(step, steps, warmup)
-    tm.update({"rows": rows, "bytes": 3 * rows * V * esize})
+    # bf16 rows of up to 155648 elements take the one-pass kernel (the row stays in a workgroup's registers): read once,
+    # written once.  Everything else is two passes: read for the row's lse, read again and written.
+    passes = 2 if (dtype_name == "bf16" and V >= 16384 and V // 8 <= 19 * 1024) else 3
+    tm.update({"rows": rows, "bytes": passes * rows * V * esize, "passes_over_the_matrix": passes,
+               "bytes_if_three_passes": 3 * rows * V * esize})
     return tm
 
 
@@ -896,9 +900,12 @@ def main():
         shapes = {}
         for rows, dn in ((4096, "bf16"), (64, "f32")):
             t = bench_full_matrix(dev, K, W, rows, dn)
-            shapes[f"{rows}x{V}_{dn}"] = {**timing_fields(t), "roofline": hbm_roofline(
+            shapes[f"{rows}x{V}_{dn}"] = {**timing_fields(t), "passes_over_the_matrix": t["passes_over_the_matrix"],
+                                          "gbs_if_priced_on_three_passes": t["bytes_if_three_passes"] / (t["ms"] * 1e-3) / 1e9,
+                                          "roofline": hbm_roofline(
                 t["bytes"], t["ms"], traffic_of(f"full_log_softmax_{rows}rows_{dn}"),
-                "row_logprob_kernel (lse) + full_log_softmax_kernel")}
+                "full_log_softmax_onepass_kernel" if t["passes_over_the_matrix"] == 2 else
+                "row_logprob_kernel (lse partials) + full_log_softmax_kernel")}
             log(f"full matrix {rows} x {V} {dn}: {t['ms'] * 1e3:.1f} us, {shapes[f'{rows}x{V}_{dn}']['roofline']['frac']:.3f} of HBM peak")
             torch.cuda.empty_cache()
         big = shapes[f"4096x{V}_bf16"]
@@ -906,7 +913,8 @@ def main():
             "value": 4096 * V / (big["ms_per_step"] * 1e-3), "unit": "log-probs written/s (4096 x 151936 bf16)",
             **{k: big[k] for k in ("ms_per_step", "median_ms", "min_ms", "settle_launches")}, "dtype": "f32", "input_dtype": "bf16",
             "config": {"workload": "tome_full_log_softmax, the drop-in of fused_log_softmax (model.py:77-89): the whole log-prob matrix in the "
-                                   "input dtype; [4096, 151936] bf16 and [64, 151936] fp32 (16 rotating buffers); algorithmic bytes 3 V sizeof(T) per row",
+                                   "input dtype; [4096, 151936] bf16 (one pass: the row stays in a workgroup's registers, 2 V sizeof(T) bytes per row) "
+                                   "and [64, 151936] fp32 (the callers' dtype; two passes, 3 V sizeof(T) bytes per row; 16 rotating buffers)",
                        "shapes": shapes},
             "roofline": big["roofline"]}
         done("full_log_softmax")

@@ -21,9 +21,14 @@ hipError_t row_logprob_noalloc_launch(const void* logits, int dtype, int64_t row
                                       const int32_t* targets, const int32_t* row_valid, float temperature,
                                       float* out_lp, float* out_lse, float* out_entropy, int32_t* out_argmax,
                                       bool* too_big, hipStream_t stream);
+hipError_t row_lse_partials_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                                   float temperature, float* out_lse, void* workspace, int* splits, hipStream_t stream);
 hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t rows, int64_t V,
                                    int64_t in_stride, int64_t out_stride, float temperature,
-                                   const float* row_lse, hipStream_t stream);
+                                   float* row_lse, const void* partials, int splits, hipStream_t stream);
+bool full_log_softmax_one_pass(const void* in, const void* out, int dtype, int64_t V, int64_t in_stride, int64_t out_stride);
+hipError_t full_log_softmax_onepass_launch(const void* in, void* out, int64_t rows, int64_t V, int64_t in_stride,
+                                           int64_t out_stride, float temperature, float* row_lse, hipStream_t stream);
 hipError_t row_sample_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
                              const float* uniforms, const int32_t* row_valid, float temperature, int top_k,
                              int32_t* out_token, float* out_lp, float* out_lse, int32_t* out_argmax,
@@ -193,11 +198,22 @@ int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows
   if (bad_temperature(temperature)) return TOME_E_TEMPERATURE;
   if (rows == 0) return TOME_OK;
   if (!logits || !out || !row_lse) return TOME_E_NULL;
-  const int rc = tome_row_logprob(logits, dtype, rows, V, in_row_stride, nullptr, nullptr, temperature, nullptr,
-                                  row_lse, nullptr, nullptr, workspace, workspace_bytes, stream);
-  if (rc != TOME_OK) return rc;
-  return hip_result(tome::full_log_softmax_launch(logits, out, dtype, rows, V, in_row_stride, out_row_stride,
-                                                  temperature, row_lse, static_cast<hipStream_t>(stream)));
+  const size_t need = tome_row_logprob_workspace(rows, V);
+  if (need > 0 && (!workspace || workspace_bytes < need)) return TOME_E_WORKSPACE;
+  const int esize = dtype == TOME_F32 ? 4 : 2;
+  if (reinterpret_cast<uintptr_t>(logits) % esize != 0 || reinterpret_cast<uintptr_t>(out) % esize != 0) return TOME_E_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // bf16 rows that fit one workgroup's registers: read once, written once
+  if (tome::full_log_softmax_one_pass(logits, out, dtype, V, in_row_stride, out_row_stride))
+    return hip_result(tome::full_log_softmax_onepass_launch(logits, out, rows, V, in_row_stride, out_row_stride, temperature,
+                                                            row_lse, s));
+  // otherwise two passes: the rows' logsumexp (split rows leave their partials in the workspace), then the matrix
+  int splits = 1;
+  const hipError_t e = tome::row_lse_partials_launch(logits, dtype, rows, V, in_row_stride, temperature, row_lse, workspace,
+                                                     &splits, s);
+  if (e != hipSuccess) return hip_result(e);
+  return hip_result(tome::full_log_softmax_launch(logits, out, dtype, rows, V, in_row_stride, out_row_stride, temperature,
+                                                  row_lse, workspace, splits, s));
 }
 
 static int check_fused(const void* hidden, const void* w, int64_t n_tokens, int64_t H, int64_t V,

@@ -3,8 +3,13 @@
 // The reference kernel (mlx-impl/model.py:57-65) computes the difference in the I/O dtype T:
 // both operands are first cast to T, and for bf16 the result is rounded once more.  The row
 // logsumexp comes from row_logprob_kernel, so the matrix is read twice and written once
-// where the reference reads it three times.
-#include "common.hpp"
+// where the reference reads it three times.  Rows that row_logprob_kernel split over several
+// workgroups are merged here, by every workgroup of the row for itself (a few partials), which
+// saves the launch of a merge kernel between the two passes.
+//
+// bf16 rows of up to 155648 elements do not need the second read either: a 1024-lane workgroup
+// holds such a row in its registers (full_log_softmax_onepass_kernel, below).
+#include "row_common.hpp"
 
 namespace tome {
 
@@ -14,7 +19,10 @@ constexpr int kFullUnroll = 4;
 struct FullArgs {
   const void* in;
   void* out;
-  const float* row_lse;
+  float* row_lse;              // read when splits == 1; written (by the row's first workgroup) otherwise
+  const RowPartial* partials;  // [rows, splits] when splits > 1
+  int splits;
+  float scale;                 // log2(e) / temperature, as the pass that made the partials used it
   int64_t V;
   int64_t in_stride;
   int64_t out_stride;
@@ -35,7 +43,26 @@ template <bool BF16, bool VECTOR>
 __global__ __launch_bounds__(kFullWG) void full_log_softmax_kernel(FullArgs a) {
   const int64_t r = blockIdx.x / a.chunks;
   const int chunk = blockIdx.x % a.chunks;
-  const float lse = a.row_lse[r];
+  float lse;
+  if (a.splits > 1) {  // merge the row's partials (at most 64: one per lane of wave 0)
+    __shared__ float lse_sh;
+    if (threadIdx.x < 64) {
+      RowStat st = stat_identity();
+      if ((int)threadIdx.x < a.splits) {
+        const RowPartial p = a.partials[r * a.splits + threadIdx.x];
+        st = RowStat{p.mx, p.s, p.w, p.bi};
+      }
+      stat_wave_reduce(st, a.scale);
+      if (threadIdx.x == 0) {
+        lse_sh = (st.mx * a.scale + fast_log2(st.s)) * kLn2;  // as finish_row forms it
+        if (chunk == 0) a.row_lse[r] = lse_sh;
+      }
+    }
+    __syncthreads();
+    lse = lse_sh;
+  } else {
+    lse = a.row_lse[r];
+  }
   constexpr int kElem = BF16 ? 2 : 4;
   constexpr int kVec = VECTOR ? 16 / kElem : 1;
   const char* in_row = static_cast<const char*>(a.in) + r * a.in_stride * kElem;
@@ -91,9 +118,134 @@ __global__ __launch_bounds__(kFullWG) void full_log_softmax_kernel(FullArgs a) {
   }
 }
 
+// ---- one pass for bf16 rows that fit a workgroup's registers ----------------------------------------
+// A 1024-lane workgroup (one per CU) loads a whole row - up to CH 16-byte units per lane, all in flight together -
+// takes the row's maximum and sum from the registers (two sweeps, as the sampler's cached variant does) and writes
+// T(x * inv_temp) - T(lse) from the same registers: the matrix is read ONCE and written once.
+template <int CH>
+__global__ __launch_bounds__(1024) void full_log_softmax_onepass_kernel(FullArgs a) {
+  constexpr int kWaves = 16;
+  __shared__ float red_m[kWaves], red_s[kWaves];
+  const int64_t r = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint16_t* in_row = static_cast<const uint16_t*>(a.in) + r * a.in_stride;
+  uint16_t* out_row = static_cast<uint16_t*>(a.out) + r * a.out_stride;
+  const u32x4* src = reinterpret_cast<const u32x4*>(in_row);
+  u32x4* dst = reinterpret_cast<u32x4*>(out_row);
+  const int n_units = (int)(a.V / 8);
+  const int n_tail = (int)(a.V - (int64_t)n_units * 8);  // single elements after the last whole unit: lane 0
+  u32x4 v[CH];
+#pragma unroll
+  for (int q = 0; q < CH; ++q) {  // unconditional (clamped) loads; unit 0 exists (checked on the host)
+    const int u = tid + q * 1024;
+    v[q] = __builtin_nontemporal_load(src + (u < n_units ? u : 0));
+  }
+  float tail[7];
+#pragma unroll
+  for (int e = 0; e < 7; ++e) tail[e] = (tid == 0 && e < n_tail) ? bf16_bits_to_f32(in_row[(int64_t)n_units * 8 + e]) : -INFINITY;
+  float m = -INFINITY;
+#pragma unroll
+  for (int q = 0; q < CH; ++q)
+    if (tid + q * 1024 < n_units) {
+      float x[8];
+      Elem<uint16_t>::unpack(v[q], x);
+      m = fmaxf(m, max_of<8>(x));
+    }
+#pragma unroll
+  for (int e = 0; e < 7; ++e) m = fmaxf(m, tail[e]);
+  m = fmaxf(m, wave_exchange<0>(m));
+  m = fmaxf(m, wave_exchange<1>(m));
+  m = fmaxf(m, wave_exchange<2>(m));
+  m = fmaxf(m, wave_exchange<3>(m));
+  m = fmaxf(m, wave_exchange<4>(m));
+  m = fmaxf(m, wave_exchange<5>(m));
+  if (lane == 0) red_m[wave] = m;
+  __syncthreads();
+  float mx = red_m[0];
+#pragma unroll
+  for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, red_m[w]);
+  mx = fmaxf(mx, kMaxFloor);  // the floor of the running maximum that every kernel of this path shares
+  const float mm = mx * a.scale;
+  float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+  for (int q = 0; q < CH; ++q)
+    if (tid + q * 1024 < n_units) {
+      float x[8];
+      Elem<uint16_t>::unpack(v[q], x);
+#pragma unroll
+      for (int i = 0; i < 8; i += 2) {
+        s0 += fast_exp2(fmaf(x[i], a.scale, -mm));
+        s1 += fast_exp2(fmaf(x[i + 1], a.scale, -mm));
+      }
+    }
+#pragma unroll
+  for (int e = 0; e < 7; ++e) s0 += fast_exp2(fmaf(tail[e], a.scale, -mm));  // -inf adds nothing
+  float ws = s0 + s1;
+  ws += wave_exchange<0>(ws);
+  ws += wave_exchange<1>(ws);
+  ws += wave_exchange<2>(ws);
+  ws += wave_exchange<3>(ws);
+  ws += wave_exchange<4>(ws);
+  ws += wave_exchange<5>(ws);
+  if (lane == 0) red_s[wave] = ws;
+  __syncthreads();
+  float sum = 0.f;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) sum += red_s[w];
+  const float lse = (mm + fast_log2(sum)) * kLn2;
+  if (tid == 0) a.row_lse[r] = lse;
+  const float lse_t = bf16_rt(lse);
+#pragma unroll
+  for (int q = 0; q < CH; ++q) {
+    const int u = tid + q * 1024;
+    if (u < n_units) {
+      u32x4 o;
+      o.x = sub_pack_bf16(v[q].x, a.inv_temp, lse_t);
+      o.y = sub_pack_bf16(v[q].y, a.inv_temp, lse_t);
+      o.z = sub_pack_bf16(v[q].z, a.inv_temp, lse_t);
+      o.w = sub_pack_bf16(v[q].w, a.inv_temp, lse_t);
+      __builtin_nontemporal_store(o, dst + u);
+    }
+  }
+  if (tid == 0)
+    for (int e = 0; e < n_tail; ++e)
+      out_row[(int64_t)n_units * 8 + e] = f32_to_bf16_bits(__fsub_rn(bf16_rt(__fmul_rn(tail[e], a.inv_temp)), lse_t));
+}
+
+constexpr int kOnePassUnits = 19;  // 16-byte units per lane: 1024 lanes hold 155648 bf16 elements
+
+// Whether the one-pass kernel takes this call: bf16, 16-byte aligned rows, a row that fits the registers of one
+// workgroup and is long enough to keep most of its 1024 lanes busy.
+bool full_log_softmax_one_pass(const void* in, const void* out, int dtype, int64_t V, int64_t in_stride, int64_t out_stride) {
+  const bool aligned = reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                       in_stride % 8 == 0 && out_stride % 8 == 0;
+  return dtype == 1 && aligned && V >= 16384 && V / 8 <= (int64_t)kOnePassUnits * 1024;
+}
+
+hipError_t full_log_softmax_onepass_launch(const void* in, void* out, int64_t rows, int64_t V, int64_t in_stride,
+                                           int64_t out_stride, float temperature, float* row_lse, hipStream_t stream) {
+  FullArgs a{};
+  a.in = in;
+  a.out = out;
+  a.row_lse = row_lse;
+  a.splits = 1;
+  a.scale = kLog2e / temperature;
+  a.V = V;
+  a.in_stride = in_stride;
+  a.out_stride = out_stride;
+  a.chunks = 1;
+  a.inv_temp = 1.0f / temperature;
+  const dim3 grid((unsigned)rows), block(1024);
+  if (V / 8 <= 8 * 1024) hipLaunchKernelGGL((full_log_softmax_onepass_kernel<8>), grid, block, 0, stream, a);
+  else hipLaunchKernelGGL((full_log_softmax_onepass_kernel<kOnePassUnits>), grid, block, 0, stream, a);
+  return hipGetLastError();
+}
+
+// Second pass.  `splits` > 1: the rows' partials (RowPartial [rows, splits]) are merged here and the merged lse is
+// also written to row_lse; splits == 1: row_lse already holds it.
 hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t rows, int64_t V,
                                    int64_t in_stride, int64_t out_stride, float temperature,
-                                   const float* row_lse, hipStream_t stream) {
+                                   float* row_lse, const void* partials, int splits, hipStream_t stream) {
   const int esize = dtype == 0 ? 4 : 2;
   const int vec = 16 / esize;
   const bool vector_ok = reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
@@ -102,6 +254,9 @@ hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t
   a.in = in;
   a.out = out;
   a.row_lse = row_lse;
+  a.partials = static_cast<const RowPartial*>(partials);
+  a.splits = splits;
+  a.scale = kLog2e / temperature;
   a.V = V;
   a.in_stride = in_stride;
   a.out_stride = out_stride;

@@ -72,16 +72,24 @@ __device__ __forceinline__ float absorb(RowStat& st, const float (&x)[N], int un
   return cm;
 }
 
-// Workgroup reduction of the per-lane states; the result is valid in every lane of wave 0.
-// Fields go through LDS one by one: a whole-struct copy to LDS leaves a private stack slot behind.
-struct RowLds {
-  float mx[kRowWaves], s[kRowWaves], w[kRowWaves];
-  int bi[kRowWaves];
+// What a workgroup leaves in the workspace when a row is split over several of them: one per (row, split).
+struct RowPartial {
+  float mx, s, w;
+  int bi;
 };
 
-// Workgroup reduction; the result is valid in wave 0 (every lane).
-__device__ __forceinline__ RowStat block_reduce(RowStat st, float scale, RowLds& lds) {
-  constexpr int kWaves = kRowWaves;
+// Workgroup reduction of the per-lane states; the result is valid in every lane of wave 0.
+// Fields go through LDS one by one: a whole-struct copy to LDS leaves a private stack slot behind.
+template <int WAVES>
+struct RowLdsT {
+  float mx[WAVES], s[WAVES], w[WAVES];
+  int bi[WAVES];
+};
+typedef RowLdsT<kRowWaves> RowLds;
+
+// Workgroup reduction (WAVES waves, at most 64); the result is valid in wave 0 (every lane).
+template <int WAVES>
+__device__ __forceinline__ RowStat block_reduce(RowStat st, float scale, RowLdsT<WAVES>& lds) {
   stat_wave_reduce(st, scale);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (lane == 0) {
@@ -93,7 +101,7 @@ __device__ __forceinline__ RowStat block_reduce(RowStat st, float scale, RowLds&
   __syncthreads();
   RowStat r = stat_identity();
   if (wave == 0) {
-    if (lane < kWaves) r = RowStat{lds.mx[lane], lds.s[lane], lds.w[lane], lds.bi[lane]};
+    if (lane < WAVES) r = RowStat{lds.mx[lane], lds.s[lane], lds.w[lane], lds.bi[lane]};
     stat_wave_reduce(r, scale);
   }
   return r;

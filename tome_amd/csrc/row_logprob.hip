@@ -18,11 +18,6 @@
 
 namespace tome {
 
-struct RowPartial {  // one per (row, split) in the workspace
-  float mx, s, w;
-  int bi;
-};
-
 // A launch scores `problems`: problem i reads row i of the logits - or, with a row list, row row_index[i] - and
 // owns entry i of targets, row_valid, the outputs and the partials.
 struct RowArgs {
@@ -203,11 +198,11 @@ __global__ __launch_bounds__(64) void row_combine_kernel(RowArgs a) {
 }
 
 template <typename T, bool VECTOR, bool ENT, bool AMAX>
-static hipError_t launch_row(const RowArgs& a, int64_t rows, hipStream_t stream) {
+static hipError_t launch_row(const RowArgs& a, int64_t rows, hipStream_t stream, bool skip_combine = false) {
   hipLaunchKernelGGL((row_logprob_kernel<T, VECTOR, ENT, AMAX>), dim3((unsigned)(rows * a.splits)),
                      dim3(kRowWG), 0, stream, a);
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess || a.splits == 1) return e;
+  if (e != hipSuccess || a.splits == 1 || skip_combine) return e;
   hipLaunchKernelGGL((row_combine_kernel<T, VECTOR, ENT, AMAX>), dim3((unsigned)rows), dim3(64), 0,
                      stream, a);
   return hipGetLastError();
@@ -267,6 +262,32 @@ hipError_t row_logprob_launch_rows(const void* logits, int dtype, int64_t n_rows
   }
   return vector_ok ? dispatch_flags<uint16_t, true>(a, rows, stream)
                    : dispatch_flags<uint16_t, false>(a, rows, stream);
+}
+
+// The rows' logsumexp for a caller that merges split rows itself: only the main kernel is launched.  With
+// *splits == 1 out_lse holds the result; otherwise the workspace holds *splits partials per row (RowPartial) and
+// out_lse is untouched.
+hipError_t row_lse_partials_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
+                                   float temperature, float* out_lse, void* workspace, int* splits, hipStream_t stream) {
+  const int esize = dtype == 0 ? 4 : 2;
+  const int vec = 16 / esize;
+  const bool vector_ok = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && (row_stride % vec == 0);
+  RowArgs a{};
+  a.logits = logits;
+  a.n_rows = rows;
+  a.out_lse = out_lse;
+  a.partials = static_cast<RowPartial*>(workspace);
+  a.V = V;
+  a.row_stride = row_stride;
+  a.splits = row_splits_for(rows, V, vector_ok ? vec : 1);
+  a.scale = kLog2e / temperature;
+  *splits = a.splits;
+  if (dtype == 0) {
+    return vector_ok ? launch_row<float, true, false, false>(a, rows, stream, true)
+                     : launch_row<float, false, false, false>(a, rows, stream, true);
+  }
+  return vector_ok ? launch_row<uint16_t, true, false, false>(a, rows, stream, true)
+                   : launch_row<uint16_t, false, false, false>(a, rows, stream, true);
 }
 
 hipError_t row_logprob_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,

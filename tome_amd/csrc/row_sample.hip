@@ -95,7 +95,8 @@ __device__ __forceinline__ int wave_rank(uint64_t key, int m) {
 // the two LDS buffers; both are clobbered.  All lanes of the workgroup must call it.
 //
 // Up to 256 keys are ranked directly: lane i counts the keys larger than key i (uniform LDS
-// addresses: broadcast reads).  More than that are first thinned by a lower bound of the k-th
+// addresses: broadcast reads; a wave none of whose lanes holds a key skips the count - the chain of a
+// decode-sized launch is bound by the instructions its waves issue, not by their latencies).  More than that are first thinned by a lower bound of the k-th
 // largest from a sample: every wave ranks 64 keys of its own (256 distinct positions spread over the
 // buffer), and the smallest of the four ceil(k/4)-th largest has >= k sampled keys at or above it;
 // at least 32 sampled keys fall below it, so every round makes progress.
@@ -130,7 +131,8 @@ __device__ uint64_t select_top_k(Lds& sh, uint64_t* cur, uint64_t* other, int m,
   if (m > kRowWG) m = kRowWG;  // unreachable, see above
   const uint64_t key = tid < m ? cur[tid] : 0;
   int rank = 0;
-  for (int j = 0; j < m; ++j) rank += cur[j] > key ? 1 : 0;
+  if (wave * 64 < m)  // wave-uniform: a wave whose lanes hold no key has nothing to rank
+    for (int j = 0; j < m; ++j) rank += cur[j] > key ? 1 : 0;
   if (tid < kSampMaxK) sh.top[tid] = 0;
   __syncthreads();
   if (key != 0 && rank < k) sh.top[rank] = key;
