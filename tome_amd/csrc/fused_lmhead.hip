@@ -1314,6 +1314,9 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   p.kind = kGeneric;
   p.small_nbt = p.small_ksteps = p.small_waves = 0;
   p.dma_nbt = n_tokens > 128 ? 4 : (n_tokens > 64 ? 2 : 1);
+  // 257 .. 384 tokens: three 128-token tiles do the MFMA work of 384 tokens where two 256-token tiles do that of 512
+  // (measured at 384 x 1024: 125 against 139 us; at 512 tokens the 256-token tile wins again, 145 against 166 us).
+  if (n_tokens > 256 && n_tokens <= 384) p.dma_nbt = 2;
   p.unit32 = 8;   // 32-row blocks per vocab unit: whole 256-row tiles unless the DMA kernel is given something finer below
   if (H % k2BK == 0) p.kind = kDma;
   // The streaming kernel runs one workgroup per CU: without a CU count (no device) the tiled kernels serve.
