@@ -26,6 +26,12 @@
  *   out_*            float32 per row; any of out_lse / out_entropy / out_argmax may
  *                    be NULL.  lse and entropy are in nats of the temperature-scaled
  *                    logits z = x / temperature.
+ *   special values   -inf logits (a masked vocabulary) carry no probability and nothing to the
+ *                    entropy; a -inf target scores -inf.  A NaN logit (or hidden state) makes that
+ *                    row's lse, lp and entropy NaN and leaves other rows alone.  The running maximum
+ *                    starts at -1e30, the floor of the reference's kernel (mlx-impl/model.py:28): a row
+ *                    whose maximum lies below it (or that holds -inf only) is outside the domain and
+ *                    comes back as lse = -inf, argmax 0, lp = +inf (NaN when the target logit is -inf).
  */
 #ifndef TOME_LOGPROB_H
 #define TOME_LOGPROB_H
@@ -143,7 +149,10 @@ int tome_row_sample(const void* logits, int dtype, int64_t rows, int64_t V, int6
  * fused_log_softmax(logits, temperature) as the reference returns it
  * (mlx-impl/model.py:77-89): out[r, j] = T(x[r, j] * (1/temp)) - T(lse_r), same shape
  * and dtype as the input, the subtraction carried out in the I/O dtype (model.py:57,60).
- * `row_lse` is a caller-provided float32 scratch of `rows` elements.
+ * `row_lse` is a caller-provided float32 buffer of `rows` elements (it receives the rows' lse);
+ * workspace: tome_row_logprob_workspace(rows, V).  bf16 rows of 16384 .. 155648 elements with
+ * 16-byte aligned rows are read once and written once (the row stays in one workgroup's registers);
+ * everything else is read twice and written once, where the reference reads three times.
  */
 int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows, int64_t V,
                           int64_t in_row_stride, int64_t out_row_stride, float temperature,

@@ -242,3 +242,49 @@ def test_row_list_matches_full_call_and_oracle(dev, dtype, rows, V, n_index):
     np.testing.assert_allclose(lp[ok], dense.lp.cpu().numpy(), atol=2e-6, rtol=0)
     np.testing.assert_array_equal(am[ok], dense.argmax.cpu().numpy())
 
+
+
+@pytest.mark.parametrize("rows,V,T", [(300, 20000, 1.0), (7, 151941, 0.7), (2, 155648, 1.0), (2, 155656, 1.3), (3, 16384, 2.0),
+                                      (5, 16376, 1.0)])
+def test_full_log_softmax_bf16_one_pass_and_its_limits(dev, rows, V, T):
+    """bf16 rows of 16384 .. 155648 elements take the one-pass kernel (the row stays in a workgroup's registers); shorter and
+    longer rows, and rows that are not 16-byte aligned, take the two passes.  Same bar for all: the bf16 arithmetic of
+    mlx-impl/model.py:57-60 as the oracle restates it, identical except where the fp32 lse sits within rounding of a bf16
+    tie; ragged V (V % 8 != 0), rows with -inf entries and a NaN row included."""
+    rng = np.random.default_rng(rows * 7 + V)
+    x32 = (rng.standard_normal((rows, V)) * 2).astype(np.float32)
+    x32[0, rng.random(V) < 0.2] = -np.inf                      # a masked vocabulary
+    if rows > 2:
+        x32[2, V // 3] = np.nan                                # NaN makes the whole row NaN
+    x = torch.from_numpy(x32).to(dev).to(torch.bfloat16)
+    out = tome_amd.fused_log_softmax(x, T)
+    assert out.shape == x.shape and out.dtype == torch.bfloat16
+    bits = bf16_bits_of(x)
+    ok = np.array([r for r in range(rows) if not (rows > 2 and r == 2)])
+    want = oracle.fused_log_softmax_f32(bits[ok], T)
+    got = bf16_bits_of(out)
+    a, b = oracle.bf16_to_f32(got[ok]), oracle.bf16_to_f32(want)
+    fin = np.isfinite(b)
+    np.testing.assert_array_equal(np.isneginf(a), np.isneginf(b))    # masked entries stay -inf
+    diff = np.abs(a[fin] - b[fin])
+    assert (diff <= 0.125 + 1e-6).all() and (diff == 0).mean() > 0.99
+    if rows > 2:
+        assert np.isnan(oracle.bf16_to_f32(got[2])).all()
+    # a strided input and output view give the same bits as the contiguous call
+    wide_in = torch.zeros((rows, V + 24), dtype=torch.bfloat16, device=dev)
+    wide_in[:, 8:V + 8] = x
+    out2 = tome_amd.fused_log_softmax(wide_in[:, 8:V + 8], T)
+    assert torch.equal(out2.view(torch.int16), out.view(torch.int16))
+
+
+def test_full_log_softmax_fp32_split_rows_merge_inside_the_second_pass(dev):
+    """fp32 batches of fewer than 512 rows are split over several workgroups in the first pass; the second pass merges
+    the partials itself.  Against the fp64 oracle at 1e-4, and the lse it leaves must equal token_logprobs' lse."""
+    rng = np.random.default_rng(123)
+    for rows, V in ((64, V_QWEN3), (9, 50001), (511, 6000)):
+        x = torch.from_numpy((rng.standard_normal((rows, V)) * 2).astype(np.float32)).to(dev)
+        out = tome_amd.fused_log_softmax(x, 0.8)
+        want = oracle.full_log_softmax64(x.cpu().numpy(), 0.8)
+        np.testing.assert_allclose(out.cpu().numpy(), want, atol=TOL_F32, rtol=0)
+        lse = tome_amd.token_logprobs(x, torch.zeros(rows, dtype=torch.int32, device=dev), 0.8, want_lse=True).lse
+        np.testing.assert_allclose((x[:, 0] / 0.8 - out[:, 0]).cpu().numpy(), lse.cpu().numpy(), atol=2e-5, rtol=0)
