@@ -5,8 +5,11 @@ A step is one pass of the hot path over one batch of synthetic input that is alr
 HBM.  The headline workload is benchmark configuration 2 (the Qwen3-0.6B GRPO ref-logprob shape:
 bf16 logits [8 x 512, 151936] with a padding mask).  The same JSON line carries one object per
 further workload: configuration 2 without its mask, configuration 1 (64 x 151936 fp32, the
-CPU-comparison shape), the fused lm_head + log-softmax kernel at configurations 3, 4 and 5, the same
-entry at decode-step and small-batch sizes, one decode step's sampler, and the LoRA merge of one
+CPU-comparison shape), the whole `process_ref_logprobs_batched` call on configuration 2's batch
+(`ref_entry`, logits and hidden-state mode: wall time per call, the kernels' share of it, host time per
+chunk), the full-matrix log-softmax drop-in, the fused lm_head + log-softmax kernel at configurations
+3, 4 and 5, the same entry behind the final RMSNorm and as the policy + reference pair over a shared
+lm_head, at decode-step and small-batch sizes, one decode step's sampler, and the LoRA merge of one
 UpdateWeights request.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only LEG[,LEG...]]
