@@ -176,8 +176,9 @@ int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows
  */
 /* Testing and tuning hook, no counterpart in the reference: kind 0 / 1 makes the fused entry points take
  * the generic / LDS-DMA sweep kernel wherever its shape rules allow, 3 the LDS-DMA kernel with every vocab
- * range cut at whole 256-row tiles (no 224-row tiles, no mixed tile heights), -1 (the default, also for any
- * other value) picks by shape.  Process-wide; set it while no call of this library is running; not for
+ * range cut at whole 256-row tiles (no 224-row tiles, no mixed tile heights), 4 / 5 the LDS-DMA kernel with its
+ * 256-token tile on two / three W buffers whatever the shape, -1 (the default, also for any other value)
+ * picks by shape.  Process-wide; set it while no call of this library is running; not for
  * production callers. */
 void tome_select_fused_kernel(int kind);
 size_t tome_fused_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V);

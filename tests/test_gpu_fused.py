@@ -20,7 +20,8 @@ def force_kernel():
     """tome_select_fused_kernel for one test: 'generic' / 'dma' force that sweep kernel, 'dma_whole_tiles' the LDS-DMA
     kernel with vocab ranges cut at whole 256-row tiles (no short last tile); reset afterwards."""
     lib = tome_amd.load_library()
-    yield lambda kind: lib.tome_select_fused_kernel({"generic": 0, "dma": 1, "dma_whole_tiles": 3}[kind])
+    yield lambda kind: lib.tome_select_fused_kernel({"generic": 0, "dma": 1, "dma_whole_tiles": 3, "dma_two_w_buffers": 4,
+                                                     "dma_three_w_buffers": 5}[kind])
     lib.tome_select_fused_kernel(-1)
 
 
@@ -252,6 +253,40 @@ def test_fused_tile_heights_agree(dev, n, H, V, force_kernel):
         assert r.lp.cpu().numpy()[n // 3] == 0 and r.argmax.cpu().numpy()[n // 3] == -1
         got[kind] = r.argmax.cpu().numpy()
     np.testing.assert_array_equal(got["dma"], got["dma_whole_tiles"])
+
+
+@pytest.mark.parametrize("n,H,V,outputs", [
+    (200, 256, 30000, "all"),       # one token tile, 224-row tiles
+    (200, 64, 3000, "plain"),       # a single K slab per vocab tile: the ring wraps at every tile
+    (700, 192, 12000, "all"),       # three token tiles, several vocab tiles per workgroup
+    (700, 192, 12000, "plain"),
+    (256, 1024, 20000, "entropy"),
+    (1500, 128, 256 * 9 + 77, "argmax"),
+])
+def test_fused_w_ring_depths_agree(dev, n, H, V, outputs, force_kernel):
+    """The 256-token tile of the LDS-DMA kernel exists with two and with three W buffers (the shape picks one): the
+    request schedule differs, the arithmetic does not, so both must match the oracle and each other bit for bit."""
+    h, w, t = _inputs(dev, n, H, V, seed=n + H, w_scale=0.1)
+    t[:4] = [0, V - 1, V // 2, 255]
+    want = oracle.lmhead_stats(bf16_bits_of(h), bf16_bits_of(w), t, 1.1)
+    ent, am = outputs in ("all", "entropy"), outputs in ("all", "argmax")
+    got = {}
+    for kind in ("dma_two_w_buffers", "dma_three_w_buffers"):
+        force_kernel(kind)
+        r = tome_amd.fused_lmhead_logprobs(h, w, torch.from_numpy(t).to(dev), 1.1, want_lse=True, want_entropy=ent, want_argmax=am)
+        np.testing.assert_allclose(r.lp.cpu().numpy(), want["lp"], atol=TOL, rtol=0)
+        np.testing.assert_allclose(r.lse.cpu().numpy(), want["lse"], atol=TOL, rtol=0)
+        if ent:
+            np.testing.assert_allclose(r.entropy.cpu().numpy(), want["entropy"], atol=TOL, rtol=0)
+        if am:
+            check_argmax(h, w, r.argmax.cpu().numpy(), want, 1.1, min_clear=0.0)
+        got[kind] = r
+    a, b = got["dma_two_w_buffers"], got["dma_three_w_buffers"]
+    assert torch.equal(a.lp, b.lp) and torch.equal(a.lse, b.lse)
+    if ent:
+        assert torch.equal(a.entropy, b.entropy)
+    if am:
+        assert torch.equal(a.argmax, b.argmax)
 
 
 @pytest.mark.parametrize("kind", ["generic", "dma", "dma_whole_tiles"])

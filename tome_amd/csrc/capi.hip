@@ -237,7 +237,7 @@ static int check_fused(const void* hidden, const void* w, int64_t n_tokens, int6
 }
 
 void tome_select_fused_kernel(int kind) {
-  tome::fused_force_kernel(kind == 0 || kind == 1 || kind == 3 ? kind : -1);
+  tome::fused_force_kernel(kind == 0 || kind == 1 || (kind >= 3 && kind <= 5) ? kind : -1);
 }
 
 size_t tome_fused_lmhead_logprob_workspace(int64_t n_tokens, int64_t H, int64_t V) {

@@ -560,7 +560,11 @@ static_assert(k2Loads == 4 && k2NBV == 8, "the MFMA/DMA interleave is written fo
 constexpr int dma_tile_tokens(int nbt) { return nbt * 64; }                                   // 4 token waves x nbt x 16
 constexpr int dma_w_bytes() { return k2BV * k2RowBytes; }                                      // 32768
 constexpr int dma_h_bytes(int nbt) { return dma_tile_tokens(nbt) * k2RowBytes; }               // 32768 at nbt = 4
-constexpr int dma_lds_bytes(int nbt) { return dma_bufs(nbt) * (dma_w_bytes() + dma_h_bytes(nbt)); }  // 131072 at nbt = 4
+// DEEP (256-token tile only): a third W buffer, which is all of the CU's LDS; see the kernel.
+constexpr int dma_w_bufs(int nbt, bool deep) { return deep ? 3 : dma_bufs(nbt); }
+constexpr int dma_lds_bytes(int nbt, bool deep = false) {  // 131072 at nbt = 4, 163840 with the third W buffer
+  return dma_w_bufs(nbt, deep) * dma_w_bytes() + dma_bufs(nbt) * dma_h_bytes(nbt);
+}
 
 // Default cache policy: non-temporal requests for either operand measured 4-5 % slower.
 __device__ __forceinline__ void dma16(const char* gptr, char* lds_wave_base) {
@@ -585,10 +589,17 @@ __device__ __forceinline__ void pair_reads() {
 // (nb = 1 .. 8) runs the same pipeline with 8 * nb MFMAs per wave and step.  Its slab keeps the LDS layout of a whole
 // tile (rows 0..127 for the waves of vocab half 0, 128..255 for half 1, so fragment addresses do not change); each
 // half holds 16 * nb rows of W and the rest of its LDS rows are requested as copies of its last row and never multiplied.
-template <bool ENT, bool AMAX, int NBT, int HI>
+//
+// DEEP: the 256-token tile with THREE W buffers and two hidden buffers (160 KB, the whole LDS of a CU) for batches of one
+// token tile, where every workgroup streams W rows of its own from HBM and a step waits for them: the W half of a slab
+// is then requested two steps ahead (in the first two quarters of a step) and the hidden half, which comes from L2, one
+// step ahead (in the last quarter).  With several token tiles the workgroups that share a W stream in L2 drift apart
+// behind the deeper ring and the kernel is slower (config 3: +4 %), so the two-buffer form stays the default.
+template <bool ENT, bool AMAX, int NBT, int HI, bool DEEP = false>
 __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   static_assert((NBT == 4 && (HI == 4 || HI == 3)) || (NBT != 4 && HI == 0), "256-token tile: every vocab tile 256 (HI = 4) or 224 rows; others: mixed heights");
+  static_assert(!DEEP || NBT == 4, "the third W buffer is for the 256-token tile");
   // The 256-token tile runs at the limit of the register file: it keeps ONE tile height per launch (4 + HI blocks per wave,
   // the host picks 256 or 224 rows), because the code for two or more heights in one kernel costs it 60 and more spilled
   // registers whose reloads, at every tile change, wait for memory behind the W stream (measured with heights of 224 and
@@ -600,9 +611,10 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   constexpr int k2NBT = NBT;                        // 16-token blocks per wave
   constexpr int k2BT = dma_tile_tokens(NBT);        // tokens per workgroup
   constexpr int kWaveTok = NBT * 16;                // tokens per wave
-  constexpr int kBufs = dma_bufs(NBT);
+  constexpr int kBufs = dma_bufs(NBT);              // hidden buffers
+  constexpr int kBufsW = dma_w_bufs(NBT, DEEP);     // W buffers
   constexpr int kWBytes = dma_w_bytes(), kHBytes = dma_h_bytes(NBT);
-  constexpr int kHBase = kBufs * kWBytes;           // the hidden ring starts behind the W ring
+  constexpr int kHBase = kBufsW * kWBytes;          // the hidden ring starts behind the W ring
   constexpr int kBLoads = NBT;                      // DMA instructions per lane and slab for the hidden rows
   constexpr int k2DmaPerSlab = k2Loads + kBLoads;   // 8 at NBT = 4
   // Portions of a request (see kIssueQ4): with three buffers everything goes out in the last quarter.
@@ -611,11 +623,20 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   constexpr int kP2 = k2DmaPerSlab - kP4 - kP1;
   static_assert(kP4 >= 1 && kP1 >= 0 && kP2 >= 0 && kP1 <= 8 && kP2 <= 8, "portions of the eight instructions");
   static_assert(kBufs == 2 || kP4 == k2DmaPerSlab, "split requests are written for two buffers");
+  // Which of the eight instructions (0-3: W, 4-7: hidden) go out in the first, second and last quarter of a step.
+  // Two buffers: a request starts in the last quarter of the step that frees its buffers (W first: it has furthest to
+  // come) and ends in the second quarter of the next.  DEEP: request step + 2 as a whole inside one step, W in the first
+  // two quarters (its buffer was freed by the previous step's barrier), hidden after this step's barrier.
+  constexpr int kQ1Lo = DEEP ? 0 : kP4, kQ1Hi = DEEP ? 2 : kP4 + kP1;
+  constexpr int kQ2Lo = kQ1Hi, kQ2Hi = DEEP ? 4 : k2DmaPerSlab;
+  constexpr int kQ4Lo = DEEP ? 4 : 0, kQ4Hi = DEEP ? k2DmaPerSlab : kP4;
+  constexpr bool kDoneAfterQ4 = DEEP || kP4 == k2DmaPerSlab;
   // Requests complete in the order they were issued, so "slab s has landed" is a count of newer instructions that
   // may still be in flight.  Before a step's barrier (slab step + 1 must be there) those are the whole requests
-  // of the slabs after it; before the loop (slab 0) also the first portion of the newest request.
-  constexpr int kInFlightAtStep = (kBufs - 2) * k2DmaPerSlab;
-  constexpr int kInFlightAtStart = (kBufs - 2) * k2DmaPerSlab + kP4;
+  // of the slabs after it (DEEP: the W instructions of request step + 2); before the loop (slab 0) also the first
+  // portion of the newest request (DEEP: the whole request for slab 1).
+  constexpr int kInFlightAtStep = DEEP ? k2Loads : (kBufs - 2) * k2DmaPerSlab;
+  constexpr int kInFlightAtStart = DEEP ? k2DmaPerSlab : (kBufs - 2) * k2DmaPerSlab + kP4;
 
   const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
   const FusedSchedule sch = a.sched_dev ? *a.sched_dev : a.sched;
@@ -718,9 +739,9 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   // the request is repeated (same addresses, same buffer, identical bytes): it is issued on every step so that
   // the code has no branch and the wait counts stay static.
   auto issue_piece = [&](int piece) {
-    const unsigned buf = (unsigned)(issued < n_steps ? issued : n_steps - 1) % kBufs;
-    if (piece < k2Loads) dma16(pa[piece], smem + buf * kWBytes + wave * 1024 + piece * 8192);
-    else dma16(pb[piece - k2Loads], smem + kHBase + buf * kHBytes + wave * 1024 + (piece - k2Loads) * 8192);
+    const unsigned slab = (unsigned)(issued < n_steps ? issued : n_steps - 1);
+    if (piece < k2Loads) dma16(pa[piece], smem + (slab % kBufsW) * kWBytes + wave * 1024 + piece * 8192);
+    else dma16(pb[piece - k2Loads], smem + kHBase + (slab % kBufs) * kHBytes + wave * 1024 + (piece - k2Loads) * 8192);
   };
   auto issue_done = [&]() {
     ++issued;
@@ -739,29 +760,38 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     }
   };
   // Fragments of one K = 32 sub-step of a slab: W blocks [i0, i0 + n) or the hidden blocks.
+  // DEEP: the offsets of the second sub-step (rdA ^ 64, rdB ^ 64) are formed where they are used (the empty asm hides
+  // that they are loop invariants).  Kept in registers across the sweep they are spilled, and a reload inside a step
+  // makes the compiler wait for EVERY outstanding memory operation - the requests two slabs ahead included.
   auto read_a = [&](int slot, int ks, int i0, bf16x8 (&fa)[4], auto n) {
-    const char* slab = smem + ((unsigned)slot % kBufs) * kWBytes;
+    const char* slab = smem + ((unsigned)slot % kBufsW) * kWBytes;
+    int rd = rdA;
+    if constexpr (DEEP) asm volatile("" : "+v"(rd));
 #pragma unroll
     for (int i = 0; i < decltype(n)::value; ++i)
-      fa[i] = *reinterpret_cast<const bf16x8*>(slab + (rdA ^ (ks * 64)) + (i0 + i) * 16 * k2RowBytes);
+      fa[i] = *reinterpret_cast<const bf16x8*>(slab + (rd ^ (ks * 64)) + (i0 + i) * 16 * k2RowBytes);
   };
   auto read_b = [&](int slot, int ks, bf16x8 (&fb)[k2NBT]) {
     const char* slab = smem + kHBase + ((unsigned)slot % kBufs) * kHBytes;
+    int rd = rdB;
+    if constexpr (DEEP) asm volatile("" : "+v"(rd));
 #pragma unroll
     for (int j = 0; j < k2NBT; ++j)
-      fb[j] = *reinterpret_cast<const bf16x8*>(slab + (rdB ^ (ks * 64)) + j * 16 * k2RowBytes);
+      fb[j] = *reinterpret_cast<const bf16x8*>(slab + (rd ^ (ks * 64)) + j * 16 * k2RowBytes);
   };
 
-  // Prologue: whole requests for all buffers but the last, and the first portion of the last one's.
+  // Prologue: whole requests for all buffers but the last, and the first portion of the last one's (DEEP: slabs 0 and 1).
 #pragma unroll
-  for (int q = 0; q < kBufs - 1; ++q) {
+  for (int q = 0; q < (DEEP ? 2 : kBufs - 1); ++q) {
 #pragma unroll
     for (int piece = 0; piece < k2DmaPerSlab; ++piece) issue_piece(piece);
     issue_done();
   }
+  if constexpr (!DEEP) {
 #pragma unroll
-  for (int piece = 0; piece < kP4; ++piece) issue_piece(piece);
-  if constexpr (kP4 == k2DmaPerSlab) issue_done();
+    for (int piece = 0; piece < kP4; ++piece) issue_piece(piece);
+    if constexpr (kP4 == k2DmaPerSlab) issue_done();
+  }
   // Slab 0 has landed (this wave's share): only the requests of the later slabs may still be in flight.
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kInFlightAtStart) : "memory");
   __builtin_amdgcn_s_barrier();
@@ -809,28 +839,28 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     __builtin_amdgcn_sched_barrier(0);
     read_a(step, 0, 4, fa_hi, hi);
 #pragma unroll
-    for (int piece = kP4; piece < kP4 + kP1; ++piece) issue_piece(piece);  // second portion of the request for slab step + 1
+    for (int piece = kQ1Lo; piece < kQ1Hi; ++piece) issue_piece(piece);  // two buffers: second portion of the request for slab step + 1
     mfma_half(0, fa_lo, fb0, fresh, lo);
     if constexpr (kTuned) {
       pair_reads<2, HIB>();
-      pair_dma(std::integral_constant<int, kP1>{});
+      pair_dma(std::integral_constant<int, kQ1Hi - kQ1Lo>{});
     }
     __builtin_amdgcn_sched_barrier(0);
     read_a(step, 1, 0, fa_lo, lo);
     read_b(step, 1, fb1);
 #pragma unroll
-    for (int piece = kP4 + kP1; piece < k2DmaPerSlab; ++piece) issue_piece(piece);  // third portion
+    for (int piece = kQ2Lo; piece < kQ2Hi; ++piece) issue_piece(piece);  // third portion
     mfma_half(4, fa_hi, fb0, fresh, hi);
     if constexpr (kTuned) {
-      if constexpr (kP2 == 0) {
+      if constexpr (kQ2Hi == kQ2Lo) {
         pair_reads<2, 8>();
       } else {
         pair_reads<1, 8>();
-        pair_dma(std::integral_constant<int, kP2>{});
+        pair_dma(std::integral_constant<int, kQ2Hi - kQ2Lo>{});
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (kP4 < k2DmaPerSlab) issue_done();
+    if constexpr (!kDoneAfterQ4) issue_done();
     read_a(step, 1, 4, fa_hi, hi);
     mfma_half(0, fa_lo, fb1, std::false_type{}, lo);
     if constexpr (kTuned) pair_reads<2, HIB>();
@@ -847,14 +877,14 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
     read_a(step + 1, 0, 0, fa_lo, kFour);
     read_b(step + 1, 0, fb0);
 #pragma unroll
-    for (int piece = 0; piece < kP4; ++piece) issue_piece(piece);
+    for (int piece = kQ4Lo; piece < kQ4Hi; ++piece) issue_piece(piece);
     mfma_half(4, fa_hi, fb1, std::false_type{}, hi);
     if constexpr (kTuned) {
       pair_reads<1, 8>();
-      pair_dma(std::integral_constant<int, kP4>{});
+      pair_dma(std::integral_constant<int, kQ4Hi - kQ4Lo>{});
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (kP4 == k2DmaPerSlab) issue_done();
+    if constexpr (kDoneAfterQ4) issue_done();
     ++step;
   };
 
@@ -1244,6 +1274,7 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
 
 enum FusedKind { kGeneric = 0, kDma = 1, kSmall = 2 };
 constexpr int kForceDmaWholeTiles = 3;  // selector value: the DMA kernel with vocab ranges cut at whole 256-row tiles
+constexpr int kForceDmaTwoWBuffers = 4, kForceDmaThreeWBuffers = 5;  // the DMA kernel, its 256-token tile with two / three W buffers
 
 // Kernel selector for tests and tuning runs: -1 (the default) picks by shape, kGeneric / kDma force that
 // sweep kernel wherever its shape rules allow.  Process-wide; set it while no call is in flight.
@@ -1254,6 +1285,7 @@ struct FusedPlan {
   FusedKind kind;
   int dma_nbt;                               // kDma only: token blocks per wave (4, 2 or 1: 256, 128 or 64 tokens per tile)
   int unit32;                                // kDma only: 32-row blocks per vocab unit (1 = mixed tile heights; 7 / 8 = whole tiles of 224 / 256 rows)
+  int dma_deep;                              // kDma, 256-token tile only: three W buffers - 0 never, 1 for sweeps without entropy and argmax, 2 always
   int small_nbt, small_ksteps, small_waves;  // kSmall only
   int bt, slots;
   int n_vunits, upt;   // vocab units the splits share out, and units per 256-row tile (what a unit costs, for the schedule)
@@ -1317,13 +1349,22 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   // 257 .. 384 tokens: three 128-token tiles do the MFMA work of 384 tokens where two 256-token tiles do that of 512
   // (measured at 384 x 1024: 125 against 139 us; at 512 tokens the 256-token tile wins again, 145 against 166 us).
   if (n_tokens > 256 && n_tokens <= 384) p.dma_nbt = 2;
+  // The third W buffer (see the kernel), measured against the two-buffer form in the same runs.  One or two token tiles:
+  // 6-13 % faster with any outputs (256 x 1024: 96 -> 87 us, 256 x 4096: 338 -> 297, 512 x 4096: 534 -> 503).  More token
+  // tiles, log-probs only: 4096 x 1024 -2.3 %, 8192 x 1024 -1.5 %, 1024 x 4096 -5 %, 4096 x 4096 -1.7 %, 16384 x 2560 -2.6 %,
+  // but 8192 x 4096 +0.2 %, 32768 x 4096 +0.7 %, 65536 x 4096 +0.5..2 %.  With the entropy or the argmax the epilogue of
+  // the deeper form spills 15-37 registers around every fold and it is 2.5 % slower at 4096 x 1024, equal at K = 4096.
+  p.dma_deep = 0;
+  if (p.dma_nbt == 4) p.dma_deep = n_tokens <= 512 ? 2 : ((H < 4096 || n_tokens < 8192) ? 1 : 0);
   p.unit32 = 8;   // 32-row blocks per vocab unit: whole 256-row tiles unless the DMA kernel is given something finer below
   if (H % k2BK == 0) p.kind = kDma;
   // The streaming kernel runs one workgroup per CU: without a CU count (no device) the tiled kernels serve.
   if (small_shape(n_tokens, H, V, p.small_nbt, p.small_ksteps, p.small_waves) && small_wg_count() >= 2) p.kind = kSmall;
   const int forced = g_forced_kind.load(std::memory_order_relaxed);
   if (forced == kGeneric) p.kind = kGeneric;
-  if ((forced == kDma || forced == kForceDmaWholeTiles) && H % k2BK == 0) p.kind = kDma;
+  if ((forced == kDma || (forced >= kForceDmaWholeTiles && forced <= kForceDmaThreeWBuffers)) && H % k2BK == 0) p.kind = kDma;
+  if (forced == kForceDmaTwoWBuffers) p.dma_deep = 0;
+  if (forced == kForceDmaThreeWBuffers && p.dma_nbt == 4) p.dma_deep = 2;
   if (p.kind == kSmall) {
     // One partial per (token, workgroup); one workgroup per CU, at most 512.
     p.bt = 128;
@@ -1398,17 +1439,19 @@ size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weigh
   return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, H, V) + normed_bytes(n_tokens, H, with_norm);
 }
 
-template <bool ENT, bool AMAX, int NBT, int HI>
+template <bool ENT, bool AMAX, int NBT, int HI, bool DEEP = false>
 static void launch_dma_nbt(const FusedArgs& a, int grid, hipStream_t stream) {
   static DeviceOnce attr_set;  // opt in to > 64 KB of dynamic LDS once per instantiation and device
   if (attr_set.first_on_current_device())
-    allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI>, dma_lds_bytes(NBT));
-  hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI>), dim3((unsigned)grid), dim3(k2WG), dma_lds_bytes(NBT),
+    allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI, DEEP>, dma_lds_bytes(NBT, DEEP));
+  hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI, DEEP>), dim3((unsigned)grid), dim3(k2WG), dma_lds_bytes(NBT, DEEP),
                      stream, a);
 }
 template <bool ENT, bool AMAX>
-static void launch_dma(const FusedArgs& a, int nbt, int unit32, int grid, hipStream_t stream) {
-  if (nbt == 4 && unit32 == 7) launch_dma_nbt<ENT, AMAX, 4, 3>(a, grid, stream);   // 224-row tiles
+static void launch_dma(const FusedArgs& a, int nbt, int unit32, bool deep, int grid, hipStream_t stream) {
+  if (nbt == 4 && unit32 == 7 && deep) launch_dma_nbt<ENT, AMAX, 4, 3, true>(a, grid, stream);
+  else if (nbt == 4 && deep) launch_dma_nbt<ENT, AMAX, 4, 4, true>(a, grid, stream);
+  else if (nbt == 4 && unit32 == 7) launch_dma_nbt<ENT, AMAX, 4, 3>(a, grid, stream);   // 224-row tiles
   else if (nbt == 4) launch_dma_nbt<ENT, AMAX, 4, 4>(a, grid, stream);
   else if (nbt == 2) launch_dma_nbt<ENT, AMAX, 2, 0>(a, grid, stream);
   else launch_dma_nbt<ENT, AMAX, 1, 0>(a, grid, stream);
@@ -1447,8 +1490,8 @@ static int launch_main(const FusedArgs& a, const FusedPlan& plan, bool want_argm
     return n;  // >= 2: fused_plan only picks this kernel when it can be placed
   }
   if (plan.kind == kDma) {
-    if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.unit32, plan.grid, stream);
-    else launch_dma<ENT, false>(a, plan.dma_nbt, plan.unit32, plan.grid, stream);
+    if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.unit32, plan.dma_deep == 2, plan.grid, stream);
+    else launch_dma<ENT, false>(a, plan.dma_nbt, plan.unit32, plan.dma_deep >= (ENT ? 2 : 1), plan.grid, stream);
   } else {
     if (want_argmax) hipLaunchKernelGGL((fused_lmhead_kernel<ENT, true>), dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
     else hipLaunchKernelGGL((fused_lmhead_kernel<ENT, false>), dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);

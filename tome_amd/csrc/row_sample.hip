@@ -74,8 +74,55 @@ struct SampleLds {
   uint64_t top[kSampMaxK];
   uint64_t thr4[kRowWaves];
   int cnt;
+  int wave_cnt[kRowWaves];
   RowLds red;
 };
+
+// Wave-cooperative collection without atomics: every wave owns a quarter of a key buffer and a running count that is
+// the same in all its lanes; the lanes that pass take consecutive slots by their position among the passing lanes.
+// An LDS atomic that returns the slot costs a round trip per candidate, and those trips queue up behind each other.
+constexpr int kSampWaveCap = kSampCap / kRowWaves;
+struct WaveCollector {
+  uint64_t* region;
+  int cap;
+  int count;  // wave-uniform; keeps counting past `cap` (overflow is detected from it), nothing is stored there
+  // Must be reached by all lanes of the wave together.
+  __device__ __forceinline__ void offer(bool pass, uint64_t key) {
+    const uint64_t b = __ballot(pass);
+    if (b == 0) return;
+    const int pos = count + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(b >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b, 0u));
+    if (pass && pos < cap) region[pos] = key;
+    count += __builtin_popcountll(b);
+  }
+};
+
+// Keys of four wave regions (counts c[w], region w starting at base + w * stride) as one list: entry i.
+__device__ __forceinline__ uint64_t region_entry(const uint64_t* base, int stride, const int* c, int i) {
+  int w = 0;
+#pragma unroll
+  for (int q = 0; q < kRowWaves - 1; ++q)
+    if (w == q && i >= c[q]) {
+      i -= c[q];
+      w = q + 1;
+    }
+  return base[w * stride + i];
+}
+
+// One wave sorts up to 64 keys held one per lane (0 = none; m = number of lanes that may hold one): returns in lane i
+// the (i+1)-th largest key for i < k, 0 elsewhere.  Register traffic only (v_readlane broadcasts, one ds_permute pair).
+__device__ __forceinline__ uint64_t wave_sorted_top_k(uint64_t key, int m, int k) {
+  const uint32_t lo = (uint32_t)key, hi = (uint32_t)(key >> 32);
+  int rank = 0;
+  for (int j = 0; j < m; ++j) {
+    const uint64_t o = ((uint64_t)__builtin_amdgcn_readlane(hi, j) << 32) | (uint32_t)__builtin_amdgcn_readlane(lo, j);
+    rank += o > key ? 1 : 0;
+  }
+  const bool keep = key != 0 && rank < k;           // k <= kSampMaxK = 32: lane 63 is never a destination
+  const int dst = (keep ? rank : 63) * 4;
+  const uint32_t slo = (uint32_t)__builtin_amdgcn_ds_permute(dst, (int)(keep ? lo : 0u));
+  const uint32_t shi = (uint32_t)__builtin_amdgcn_ds_permute(dst, (int)(keep ? hi : 0u));
+  return ((uint64_t)shi << 32) | slo;               // lanes nobody sends to read 0
+}
 
 // Number of lanes of this wave whose key is larger than this lane's.  v_readlane broadcasts (the lane
 // index is uniform), not LDS-crossbar shuffles: 64 dependent ds_bpermute round trips cost microseconds.
@@ -171,12 +218,10 @@ __device__ uint64_t bound_from_lane_maxima(Lds& sh, float lane_max, int k) {
   return thr;
 }
 
-// Wave 0: draw among the sorted candidates in sh.top and write the row's outputs.  `tot` holds the
-// full-vocabulary (max, sum) in every lane.
-template <class Lds>
-__device__ __forceinline__ void finish_sample(const SampleArgs& a, Lds& sh, int64_t r, const RowStat& tot, int lane) {
+// Wave 0: draw among the sorted candidates (lane i < k holds the (i+1)-th largest key, 0 = none) and write the
+// row's outputs.  `tot` holds the full-vocabulary (max, sum) in every lane.
+__device__ __forceinline__ void finish_sample(const SampleArgs& a, uint64_t key, int64_t r, const RowStat& tot, int lane) {
   const int k = a.top_k;
-  const uint64_t key = lane < k ? sh.top[lane] : 0;
   const bool have = key != 0;
   const float x = have ? key_float((uint32_t)(key >> 32)) : -INFINITY;
   const int n_have = __builtin_popcountll(__ballot(have));
@@ -268,6 +313,7 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
   float lane_max = -INFINITY;  // this lane's largest element, or -inf when it saw nothing above -inf
   RowStat tot = stat_identity();
   uint64_t theta = 0;
+  float tail[Elem<T>::kVec - 1];  // cached variant: the single elements after the last whole unit (lane 0 of the last split)
   if constexpr (CACHED) {
     // Everything a lane owns is in registers, so the statistics take two sweeps over them instead of an online
     // update: the maxima first, then the sum of 2^(y - m) against one reference per wave (no rescaling chain).
@@ -277,7 +323,6 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
       const int64_t u = u0 + tid + q * kRowWG;
       cached[q] = p[u < u1 ? u : 0];         // unit 0 exists (checked on the host)
     }
-    float tail[Elem<T>::kVec - 1];           // single elements after the last whole unit: lane 0 of the last split
 #pragma unroll
     for (int e = 0; e < kVec - 1; ++e) tail[e] = (tid == 0 && e < n_tail) ? Elem<T>::load1(row + n_units * kVec + e) : -INFINITY;
 #pragma unroll
@@ -421,11 +466,11 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
   }
 
   // ---- pass 2: collect every element >= theta ---------------------------------------------------
-  // sh.cnt is zero here: cleared before the first barrier, and again after an overflow.
-  while (scan) {
-    const float theta_val = theta == 0 ? -INFINITY : key_float((uint32_t)(theta >> 32));
-    auto offer2 = [&](float x, int64_t idx) { offer(x, idx, theta, theta_val); };
-    if constexpr (CACHED) {
+  uint64_t sorted = 0;  // wave 0, lane i < k: the (i+1)-th largest key of this range
+  if constexpr (CACHED) {
+    // sh.cnt is zero here: cleared before the first barrier, and again after an overflow.
+    for (;;) {
+      const float theta_val = theta == 0 ? -INFINITY : key_float((uint32_t)(theta >> 32));
       // Opaque to the optimiser, so that the keys and element indices below are formed where they are
       // used (rarely) instead of being hoisted out of the retry loop into a hundred live registers.
       uint32_t first_elem = (uint32_t)((u0 + tid) * kVec);
@@ -440,63 +485,91 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
           Elem<T>::unpack(cached[q], x);
           if (max_of<kVec>(x) >= theta_val) {
 #pragma unroll
-            for (int i = 0; i < kVec; ++i) offer2(x[i], first_elem + (uint32_t)(q * kRowWG * kVec + i));
+            for (int i = 0; i < kVec; ++i) offer(x[i], first_elem + (uint32_t)(q * kRowWG * kVec + i), theta, theta_val);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
       if (tid == 0)
-        for (int e = 0; e < n_tail; ++e) offer2(Elem<T>::load1(row + n_units * kVec + e), n_units * kVec + e);
-    } else if constexpr (VECTOR) {
-      const u32x4* p = reinterpret_cast<const u32x4*>(row);
-      int64_t u = u0 + tid;
-      for (; u + (kRowUnroll - 1) * kRowWG < u1; u += kRowUnroll * kRowWG) {
-        u32x4 v[kRowUnroll];
 #pragma unroll
-        for (int q = 0; q < kRowUnroll; ++q) v[q] = p[u + q * kRowWG];
+        for (int e = 0; e < kVec - 1; ++e) offer(tail[e], n_units * kVec + e, theta, theta_val);  // -inf where there is none
+      __syncthreads();
+      const int offered = sh.cnt;
+      if (offered <= kSampCap) {
+        m = offered;
+        break;
+      }
+      // Overflow: the k-th largest of the kSampCap keys that were kept is a strictly higher lower bound.
+      __syncthreads();
+      theta = select_top_k(sh, sh.a, sh.b, kSampCap, k);
+      if (tid == 0) sh.cnt = 0;
+      __syncthreads();
+    }
+    if (m <= 64) {  // the usual case: wave 0 ranks them in registers, the other waves are done
+      if (wave != 0) return;
+      sorted = wave_sorted_top_k(lane < m ? sh.a[lane] : 0, m, k);
+    } else {
+      select_top_k(sh, sh.a, sh.b, m, k);
+      if (wave != 0) return;
+      sorted = lane < k ? sh.top[lane] : 0;
+    }
+  } else {
+    // sh.cnt is zero here: cleared before the first barrier, and again after an overflow.
+    while (scan) {
+      const float theta_val = theta == 0 ? -INFINITY : key_float((uint32_t)(theta >> 32));
+      auto offer2 = [&](float x, int64_t idx) { offer(x, idx, theta, theta_val); };
+      if constexpr (VECTOR) {
+        const u32x4* p = reinterpret_cast<const u32x4*>(row);
+        int64_t u = u0 + tid;
+        for (; u + (kRowUnroll - 1) * kRowWG < u1; u += kRowUnroll * kRowWG) {
+          u32x4 v[kRowUnroll];
 #pragma unroll
-        for (int q = 0; q < kRowUnroll; ++q) {
-          float x[kVec];
-          Elem<T>::unpack(v[q], x);
-          if (max_of<kVec>(x) >= theta_val) {
+          for (int q = 0; q < kRowUnroll; ++q) v[q] = p[u + q * kRowWG];
 #pragma unroll
-            for (int i = 0; i < kVec; ++i) offer2(x[i], (u + q * kRowWG) * kVec + i);
+          for (int q = 0; q < kRowUnroll; ++q) {
+            float x[kVec];
+            Elem<T>::unpack(v[q], x);
+            if (max_of<kVec>(x) >= theta_val) {
+#pragma unroll
+              for (int i = 0; i < kVec; ++i) offer2(x[i], (u + q * kRowWG) * kVec + i);
+            }
           }
         }
-      }
-      for (; u < u1; u += kRowWG) {
-        float x[kVec];
-        Elem<T>::unpack(p[u], x);
-        if (max_of<kVec>(x) >= theta_val) {
+        for (; u < u1; u += kRowWG) {
+          float x[kVec];
+          Elem<T>::unpack(p[u], x);
+          if (max_of<kVec>(x) >= theta_val) {
 #pragma unroll
-          for (int i = 0; i < kVec; ++i) offer2(x[i], u * kVec + i);
+            for (int i = 0; i < kVec; ++i) offer2(x[i], u * kVec + i);
+          }
         }
+        if (tid == 0)
+          for (int e = 0; e < n_tail; ++e) offer2(Elem<T>::load1(row + n_units * kVec + e), n_units * kVec + e);
+      } else {
+        for (int64_t u = u0 + tid; u < u1; u += kRowWG) offer2(Elem<T>::load1(row + u), u);
       }
-      if (tid == 0)
-        for (int e = 0; e < n_tail; ++e) offer2(Elem<T>::load1(row + n_units * kVec + e), n_units * kVec + e);
-    } else {
-      for (int64_t u = u0 + tid; u < u1; u += kRowWG) offer2(Elem<T>::load1(row + u), u);
+      __syncthreads();
+      const int offered = sh.cnt;
+      if (offered <= kSampCap) {
+        m = offered;
+        break;
+      }
+      // Overflow: the k-th largest of the kSampCap keys that were kept is a strictly higher lower bound.
+      __syncthreads();
+      theta = select_top_k(sh, sh.a, sh.b, kSampCap, k);
+      if (tid == 0) sh.cnt = 0;
+      __syncthreads();
     }
-    __syncthreads();
-    const int offered = sh.cnt;
-    if (offered <= kSampCap) {
-      m = offered;
-      break;
-    }
-    // Overflow: the k-th largest of the kSampCap keys that were kept is a strictly higher lower bound.
-    __syncthreads();
-    theta = select_top_k(sh, sh.a, sh.b, kSampCap, k);
-    if (tid == 0) sh.cnt = 0;
-    __syncthreads();
+    select_top_k(sh, sh.a, sh.b, m, k);
+    if (wave != 0) return;
+    sorted = lane < k ? sh.top[lane] : 0;
   }
 
-  // ---- final selection ---------------------------------------------------------------------------
-  select_top_k(sh, sh.a, sh.b, m, k);
-  if (wave != 0) return;
+  // ---- wave 0: the row's outputs, or this range's record for the combine kernel -----------------------
   if (a.splits == 1) {
-    finish_sample(a, sh, r, tot, lane);
+    finish_sample(a, sorted, r, tot, lane);
   } else {
     const int64_t slot = r * a.splits + split;
-    if (lane < k) a.part_keys[slot * k + lane] = sh.top[lane];
+    if (lane < k) a.part_keys[slot * k + lane] = sorted;
     if (lane == 0) a.part_stat[slot] = float2{tot.mx, tot.s};
   }
 }
@@ -509,9 +582,11 @@ __global__ __launch_bounds__(kRowWG) void row_sample_combine_kernel(SampleArgs a
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int k = a.top_k, m = a.splits * k;         // <= 64 * 32 = kSampMergeCap
   const uint64_t* keys = a.part_keys + r * m;      // per split: its k keys in descending order, 0 past the end
-  // Every key is fetched once, up front and together with the statistics: the kernel then waits for global memory
-  // one time (the previous launch wrote these bytes on other dies, so each wait is a trip beyond the L2).
+  // Every key is fetched once, up front and together with the statistics and the heads for the bound: the kernel then
+  // waits for global memory one time (the previous launch wrote these bytes on other dies, so each wait is a trip
+  // beyond the L2).
   constexpr int kPer = kSampMergeCap / kRowWG;
+  constexpr int kWaveCap = kSampMergeCap / kRowWaves;
   uint64_t mine[kPer];
 #pragma unroll
   for (int q = 0; q < kPer; ++q) {
@@ -519,46 +594,58 @@ __global__ __launch_bounds__(kRowWG) void row_sample_combine_kernel(SampleArgs a
     mine[q] = i < m ? keys[i] : 0;
   }
   RowStat st = stat_identity();
-  if (wave == 0 && lane < a.splits) {
-    const float2 p = a.part_stat[r * a.splits + lane];
-    st.mx = p.x;
-    st.s = p.y;
-  }
-  if (tid == 0) {
-    sh.thr4[0] = 0;
-    sh.cnt = 0;
-  }
-  if (m > kRowWG) {  // staged for the bound below
-#pragma unroll
-    for (int q = 0; q < kPer; ++q) {
-      const int i = tid + q * kRowWG;
-      if (i < m) sh.b[i] = mine[q];
+  uint64_t head = 0;
+  if (wave == 0) {
+    if (lane < a.splits) {
+      const float2 p = a.part_stat[r * a.splits + lane];
+      st.mx = p.x;
+      st.s = p.y;
     }
-  }
-  __syncthreads();
-  // A lower bound of the k-th largest from the heads of the lists: the largest 64 / splits keys of every
-  // split (more than k keys in all); its k-th largest keeps a few dozen of the splits * k keys.
-  if (m > kRowWG && wave == 0) {
-    const int per = 64 / a.splits;                 // >= 1: splits <= 64
-    const int sp = lane / per, j = lane % per;
-    const uint64_t key = (sp < a.splits && j < k) ? sh.b[sp * k + j] : 0;
-    const int rank = wave_rank(key, 64);
-    if (key != 0 && rank == k - 1) sh.thr4[0] = key;
+    // A lower bound of the k-th largest from the heads of the lists: the largest 64 / splits keys of every
+    // split; where those are k keys or more, their k-th largest keeps a few dozen of the splits * k keys.
+    if (m > 64) {
+      const int per = 64 / a.splits;               // >= 1: splits <= 64
+      const int sp = lane / per, j = lane % per;
+      if (sp < a.splits && j < k) head = keys[sp * k + j];
+    }
+    uint64_t thr = 0;
+    if (m > 64) {
+      const int rank = wave_rank(head, 64);
+      const uint64_t at = __ballot(head != 0 && rank == k - 1);  // at most one lane: keys are distinct
+      if (at != 0) {
+        const int src = __builtin_ctzll(at);
+        thr = ((uint64_t)__builtin_amdgcn_readlane((uint32_t)(head >> 32), src) << 32) |
+              (uint32_t)__builtin_amdgcn_readlane((uint32_t)head, src);
+      }
+    }
+    if (lane == 0) sh.thr4[0] = thr;
   }
   __syncthreads();
   const uint64_t thr = sh.thr4[0];
+  WaveCollector col{sh.a + wave * kWaveCap, kWaveCap, 0};  // a wave offers at most kPer * 64 = kWaveCap keys: no overflow
 #pragma unroll
-  for (int q = 0; q < kPer; ++q) {
-    const uint64_t key = mine[q];
-    if (key != 0 && key >= thr) sh.a[atomicAdd(&sh.cnt, 1)] = key;
+  for (int q = 0; q < kPer; ++q)
+    if (q * kRowWG + wave * 64 < m)  // wave-uniform
+      col.offer(mine[q] != 0 && mine[q] >= thr, mine[q]);
+  if (lane == 0) sh.wave_cnt[wave] = col.count;
+  __syncthreads();
+  int c[kRowWaves];
+#pragma unroll
+  for (int w = 0; w < kRowWaves; ++w) c[w] = sh.wave_cnt[w];
+  const int kept = c[0] + c[1] + c[2] + c[3];
+  uint64_t sorted;
+  if (kept <= 64) {  // the usual case: wave 0 ranks them in registers
+    if (wave != 0) return;
+    sorted = wave_sorted_top_k(lane < kept ? region_entry(sh.a, kWaveCap, c, lane) : 0, kept, k);
+  } else {
+    for (int i = tid; i < kept; i += kRowWG) sh.b[i] = region_entry(sh.a, kWaveCap, c, i);
+    __syncthreads();
+    select_top_k(sh, sh.b, sh.a, kept, k);
+    if (wave != 0) return;
+    sorted = lane < k ? sh.top[lane] : 0;
   }
-  __syncthreads();
-  const int kept = sh.cnt;
-  __syncthreads();
-  select_top_k(sh, sh.a, sh.b, kept, k);
-  if (wave != 0) return;
   stat_wave_reduce(st, a.scale);
-  finish_sample(a, sh, r, st, lane);
+  finish_sample(a, sorted, r, st, lane);
 }
 
 int row_splits_for(int64_t rows, int64_t V, int vec);
