@@ -22,7 +22,7 @@ median of the per-launch times (`median_ms`, `min_ms`; this second pass does not
 The matrix-core legs add a clock pass: the same step is queued for CLOCK_MS of GPU time (untimed) and the
 host meanwhile reads the engine clock the driver reports (`pp_dpm_sclk` of the device in sysfs, a
 smoothed value) every few milliseconds; the median of the samples from the second half of that pass
-is `sclk_mhz`, and these legs price themselves against the published peak scaled to that clock as well
+is `sclk_mhz` (with the socket power and its cap from the same device's hwmon files as `power_w`, `power_cap_w`), and these legs price themselves against the published peak scaled to that clock as well
 (`roofline.peak_at_sclk`, `roofline.frac_at_sclk`): the published 2.5 PFLOP/s is 256 CUs x 4096 FLOP per clock at the 2.4 GHz peak engine clock, which the part does not
 hold under a matrix-core load on random operands.  The `ceiling` leg times the fused kernel's LDS -> MFMA loop
 alone on random operands (`sustained_peak` in the later matrix-core legs), with the kernel's fill requests
@@ -135,6 +135,34 @@ def read_sclk_mhz():
     return None
 
 
+def power_paths():
+    """(sysfs file with the socket power in microwatts, file with its cap) of the same GPU, or (None, None)."""
+    if "power" not in _SCLK:
+        import glob
+        avg = cap = None
+        if sclk_path():
+            dev = os.path.dirname(sclk_path())
+            for name in ("power1_average", "power1_input"):
+                hits = sorted(glob.glob(os.path.join(dev, "hwmon", "hwmon*", name)))
+                if hits:
+                    avg = hits[0]
+                    break
+            hits = sorted(glob.glob(os.path.join(dev, "hwmon", "hwmon*", "power1_cap")))
+            cap = hits[0] if hits else None
+        _SCLK["power"] = (avg, cap)
+    return _SCLK["power"]
+
+
+def read_watts(path):
+    if not path:
+        return None
+    try:
+        with open(path) as f:
+            return float(f.read().strip()) / 1e6
+    except (OSError, ValueError):
+        return None
+
+
 def time_steps(fn, steps, warmup, clock=False):
     """Warm-up, settle, timed region, per-launch pass (see the module docstring).  Times in milliseconds by
     HIP events recorded on the stream the kernels run on (torch's current stream, which the library
@@ -174,7 +202,7 @@ def time_steps(fn, steps, warmup, clock=False):
         ev[i + 1].record()
     torch.cuda.synchronize()
     per = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(steps))
-    clocks = []   # clock pass: the engine clock while the same step keeps the GPU busy for CLOCK["ms"]
+    clocks, watts = [], []   # clock pass: the engine clock (and the socket power) while the same step keeps the GPU busy for CLOCK["ms"]
     if clock and CLOCK["ms"] > 0 and sclk_path():
         n = max(steps, int(CLOCK["ms"] / mean_ms) + 1)
         done = torch.cuda.Event()
@@ -184,14 +212,20 @@ def time_steps(fn, steps, warmup, clock=False):
         done.record()
         while not done.query():
             c = read_sclk_mhz()
+            w = read_watts(power_paths()[0])
             if c and not done.query():
                 clocks.append((time.perf_counter() - t1, c))
+                if w:
+                    watts.append((time.perf_counter() - t1, w))
             time.sleep(0.003)
         torch.cuda.synchronize()
         half = (time.perf_counter() - t1) / 2
         clocks = sorted(c for (at, c) in clocks if at >= half)
+        watts = sorted(w for (at, w) in watts if at >= half)
     return {"ms": mean_ms, "wall_ms": wall_ms, "median_ms": per[len(per) // 2], "min_ms": per[0],
-            "settle_launches": settle, "sclk_mhz": clocks[len(clocks) // 2] if clocks else None}
+            "settle_launches": settle, "sclk_mhz": clocks[len(clocks) // 2] if clocks else None,
+            "power_w": watts[len(watts) // 2] if watts else None,
+            "power_cap_w": read_watts(power_paths()[1]) if watts else None}
 
 
 def timing_fields(t):
@@ -199,6 +233,9 @@ def timing_fields(t):
          "settle_launches": t["settle_launches"]}
     if t.get("sclk_mhz"):
         d["sclk_mhz"] = t["sclk_mhz"]
+    if t.get("power_w"):   # socket power the driver reports during the clock pass, and the cap it regulates to
+        d["power_w"] = t["power_w"]
+        d["power_cap_w"] = t.get("power_cap_w")
     return d
 
 
