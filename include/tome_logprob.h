@@ -171,7 +171,8 @@ int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows
  *
  * Process-wide state of the library, all of it caches that do not change results and all of it kept per
  * device ordinal: the CU count (one workgroup per CU for batches of up to 128 tokens), a flag per large-LDS
- * kernel ("dynamic LDS limit raised"), the device address of tome_row_logprob_noalloc's array; and the
+ * kernel ("dynamic LDS limit raised", and "the 160 KB of the three-buffer sweep were refused": the two-buffer
+ * sweep then serves), the device address of tome_row_logprob_noalloc's array; and the
  * two testing hooks (the selector below, tome_row_logprob_noalloc_limit).
  */
 /* Testing and tuning hook, no counterpart in the reference: kind 0 / 1 makes the fused entry points take

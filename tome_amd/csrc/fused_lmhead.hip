@@ -1294,8 +1294,19 @@ struct FusedPlan {
 };
 
 template <typename K>
-static void allow_big_lds(K kernel, int bytes) {
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+static bool allow_big_lds(K kernel, int bytes) {
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess)
+    return true;
+  (void)hipGetLastError();  // the launch that follows reports its own error
+  return false;
+}
+// Devices (bit per ordinal) that did not grant the 160 KB of dynamic LDS the three-buffer form asks for - all of a CU's
+// LDS, which a driver may not hand out whole: the two-buffer form serves there.
+static std::atomic<uint64_t> g_no_deep_lds{0};
+static bool deep_lds_refused() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDeviceOrdinals) return false;
+  return (g_no_deep_lds.load(std::memory_order_relaxed) >> dev) & 1;
 }
 
 // Workgroups of the small-batch kernel: one per CU.  Measured at 16 and 64 tokens, H = 1024: 256 workgroups
@@ -1442,8 +1453,15 @@ size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weigh
 template <bool ENT, bool AMAX, int NBT, int HI, bool DEEP = false>
 static void launch_dma_nbt(const FusedArgs& a, int grid, hipStream_t stream) {
   static DeviceOnce attr_set;  // opt in to > 64 KB of dynamic LDS once per instantiation and device
-  if (attr_set.first_on_current_device())
-    allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI, DEEP>, dma_lds_bytes(NBT, DEEP));
+  if (attr_set.first_on_current_device() &&
+      !allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI, DEEP>, dma_lds_bytes(NBT, DEEP)) && DEEP) {
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDeviceOrdinals)
+      g_no_deep_lds.fetch_or(1ull << dev, std::memory_order_relaxed);
+  }
+  if constexpr (DEEP) {
+    if (deep_lds_refused()) return launch_dma_nbt<ENT, AMAX, NBT, HI, false>(a, grid, stream);
+  }
   hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI, DEEP>), dim3((unsigned)grid), dim3(k2WG), dma_lds_bytes(NBT, DEEP),
                      stream, a);
 }
