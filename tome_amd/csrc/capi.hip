@@ -26,7 +26,7 @@ hipError_t row_lse_partials_launch(const void* logits, int dtype, int64_t rows, 
 hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t rows, int64_t V,
                                    int64_t in_stride, int64_t out_stride, float temperature,
                                    float* row_lse, const void* partials, int splits, hipStream_t stream);
-bool full_log_softmax_one_pass(const void* in, const void* out, int dtype, int64_t V, int64_t in_stride, int64_t out_stride);
+bool full_log_softmax_one_pass(const void* in, const void* out, int dtype, int64_t rows, int64_t V, int64_t in_stride, int64_t out_stride);
 hipError_t full_log_softmax_onepass_launch(const void* in, void* out, int64_t rows, int64_t V, int64_t in_stride,
                                            int64_t out_stride, float temperature, float* row_lse, hipStream_t stream);
 hipError_t row_sample_launch(const void* logits, int dtype, int64_t rows, int64_t V, int64_t row_stride,
@@ -204,7 +204,7 @@ int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows
   if (reinterpret_cast<uintptr_t>(logits) % esize != 0 || reinterpret_cast<uintptr_t>(out) % esize != 0) return TOME_E_ALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   // bf16 rows that fit one workgroup's registers: read once, written once
-  if (tome::full_log_softmax_one_pass(logits, out, dtype, V, in_row_stride, out_row_stride))
+  if (tome::full_log_softmax_one_pass(logits, out, dtype, rows, V, in_row_stride, out_row_stride))
     return hip_result(tome::full_log_softmax_onepass_launch(logits, out, rows, V, in_row_stride, out_row_stride, temperature,
                                                             row_lse, s));
   // otherwise two passes: the rows' logsumexp (split rows leave their partials in the workspace), then the matrix

@@ -216,10 +216,13 @@ constexpr int kOnePassUnits = 19;  // 16-byte units per lane: 1024 lanes hold 15
 
 // Whether the one-pass kernel takes this call: bf16, 16-byte aligned rows, a row that fits the registers of one
 // workgroup and is long enough to keep most of its 1024 lanes busy.
-bool full_log_softmax_one_pass(const void* in, const void* out, int dtype, int64_t V, int64_t in_stride, int64_t out_stride) {
+// One workgroup per row leaves most of the chip idle on a decode-sized batch: below ~96 rows the two-pass kernels, which
+// split a row over several workgroups, are faster (8 / 32 / 64 rows of 151936 bf16: 7.9 / 11.6 / 16.5 us against 17.3 /
+// 18.0 / 18.5; 128 / 512 / 2048 rows: 25.4 / 77.5 / 291 against 20.1 / 63.6 / 238).
+bool full_log_softmax_one_pass(const void* in, const void* out, int dtype, int64_t rows, int64_t V, int64_t in_stride, int64_t out_stride) {
   const bool aligned = reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
                        in_stride % 8 == 0 && out_stride % 8 == 0;
-  return dtype == 1 && aligned && V >= 16384 && V / 8 <= (int64_t)kOnePassUnits * 1024;
+  return dtype == 1 && aligned && rows >= 96 && V >= 16384 && V / 8 <= (int64_t)kOnePassUnits * 1024;
 }
 
 hipError_t full_log_softmax_onepass_launch(const void* in, void* out, int64_t rows, int64_t V, int64_t in_stride,
