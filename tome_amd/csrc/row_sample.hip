@@ -650,17 +650,20 @@ __global__ __launch_bounds__(kRowWG) void row_sample_combine_kernel(SampleArgs a
 
 int row_splits_for(int64_t rows, int64_t V, int vec);
 
-// Workgroups per row.  Large batches follow the row kernel (one workgroup per row from 512 rows on).
-// Decode-sized batches are cut into ranges of ~8192 elements whatever the batch size: the selection
+// Workgroups per row.  Decode-sized batches are cut into ranges of ~8192 elements whatever the batch size: the selection
 // bookkeeping of a workgroup grows with its elements, 8192 fp32 elements are the most a workgroup keeps in
 // registers between its passes, and fewer, fatter workgroups beat filling the chip (64 rows fp32: 19-20
 // splits 23 us, 32 splits 27 us, 12 splits 37 us; 256 rows: 20 splits 47 us, the row kernel's 8 splits
-// 68 us).  Very small batches still get enough workgroups to pull a row from many CUs.
+// 68 us).  Very small batches still get enough workgroups to pull a row from many CUs.  Larger batches follow the
+// row kernel (one workgroup per row from 512 rows on, which streams the row once); where that takes over was measured
+// at V = 151936, ranges against the row kernel's policy: fp32 512 / 768 / 1024 / 1280 rows 63.9 / 89.4 / 116.3 / 145.1 us
+// against 85.0 / 97.4 / 118.8 / 143.8; bf16 300 / 350 / 400 / 512 rows 46.7 / 51.6 / 56.9 / 69.1 against 51.5 / 52.0 /
+// 54.6 / 61.5 (a bf16 range holds twice the elements per byte, and it is the per-element work that costs).
 static int sample_splits_for(int64_t rows, int64_t V, int vec) {
   const int base = row_splits_for(rows, V, vec);
-  if (base == 1) return 1;
   int64_t s = (V + 8191) / 8192;
-  if (rows * s > 8192) return base;          // hundreds of rows: the row kernel's policy
+  const int64_t most_ranges = vec == 4 ? 20000 : 6500;   // rows * ranges: ~1050 fp32 rows, ~340 bf16 rows at V = 151936
+  if (rows * s > most_ranges) return base;
   const int64_t fill = (512 + rows - 1) / rows;
   if (s < fill) s = fill;
   const int64_t max_by_work = (V / vec) / (2 * kRowWG);  // >= 2 load units per lane and split
