@@ -508,7 +508,7 @@ __device__ __forceinline__ void write_partials16(RowStat (&st)[NBT], float (&tx)
 
 // ===============================================================================================
 // Fast path (H % 64 == 0): 512 lanes, 256 x 256 tile, v_mfma_f32_16x16x32_bf16, K slabs DMA'd straight
-// into LDS, double-buffered.
+// into LDS, double-buffered (a third W buffer in the DEEP form, below).
 //
 //   * 8 waves as 2 (vocab) x 4 (token), 128 vocab x 64 tokens per wave as 8 x 4 blocks of 16x16.  The
 //     16x16x32 MFMA moves half the accumulator bytes per FLOP of the 32x32x16 one; on this
@@ -590,11 +590,13 @@ __device__ __forceinline__ void pair_reads() {
 // tile (rows 0..127 for the waves of vocab half 0, 128..255 for half 1, so fragment addresses do not change); each
 // half holds 16 * nb rows of W and the rest of its LDS rows are requested as copies of its last row and never multiplied.
 //
-// DEEP: the 256-token tile with THREE W buffers and two hidden buffers (160 KB, the whole LDS of a CU) for batches of one
-// token tile, where every workgroup streams W rows of its own from HBM and a step waits for them: the W half of a slab
-// is then requested two steps ahead (in the first two quarters of a step) and the hidden half, which comes from L2, one
-// step ahead (in the last quarter).  With several token tiles the workgroups that share a W stream in L2 drift apart
-// behind the deeper ring and the kernel is slower (config 3: +4 %), so the two-buffer form stays the default.
+// DEEP: the 256-token tile with THREE W buffers and two hidden buffers (160 KB, the whole LDS of a CU).  The W half of
+// a slab is requested two steps ahead - in the first two quarters of a step, its buffer free since the previous step's
+// barrier - and the hidden half, which comes from L2, one step ahead, after the step's own barrier; before a barrier
+// the four W instructions of the newest request stay in flight.  Faster wherever a step waits for its fill: 10-15 %
+// where every workgroup streams W rows of its own (one token tile), 2-3 % at 4096 x 1024 tokens x hidden, nothing from
+// 8192 x 4096 on; with the entropy or the argmax its fold spills and it only pays at one or two token tiles
+// (fused_plan holds the rule and the figures).
 template <bool ENT, bool AMAX, int NBT, int HI, bool DEEP = false>
 __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
