@@ -321,7 +321,7 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
 #pragma unroll
     for (int q = 0; q < kSampCached; ++q) {  // unconditional (clamped) loads: all eight in flight together
       const int64_t u = u0 + tid + q * kRowWG;
-      cached[q] = p[u < u1 ? u : 0];         // unit 0 exists (checked on the host)
+      cached[q] = __builtin_nontemporal_load(p + (u < u1 ? u : 0));  // unit 0 exists (checked on the host)
     }
 #pragma unroll
     for (int e = 0; e < kVec - 1; ++e) tail[e] = (tid == 0 && e < n_tail) ? Elem<T>::load1(row + n_units * kVec + e) : -INFINITY;
@@ -400,7 +400,7 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
     if (n_groups > 0 && big_range) {  // first iteration: statistics, then the bound, then its candidates
       u32x4 first[kRowUnroll];
 #pragma unroll
-      for (int q = 0; q < kRowUnroll; ++q) first[q] = p[u0 + tid + q * kRowWG];
+      for (int q = 0; q < kRowUnroll; ++q) first[q] = __builtin_nontemporal_load(p + u0 + tid + q * kRowWG);
 #pragma unroll
       for (int q = 0; q < kRowUnroll; ++q) {
         float x[kVec];
@@ -426,11 +426,11 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
       if (gi == g_renew) renew_bound();  // uniform: every lane runs the same iterations
       u32x4 v[kRowUnroll];
 #pragma unroll
-      for (int q = 0; q < kRowUnroll; ++q) v[q] = p[u0 + gi * kGroup + tid + q * kRowWG];
+      for (int q = 0; q < kRowUnroll; ++q) v[q] = __builtin_nontemporal_load(p + u0 + gi * kGroup + tid + q * kRowWG);
 #pragma unroll
       for (int q = 0; q < kRowUnroll; ++q) consume(v[q], u0 + gi * kGroup + tid + q * kRowWG);
     }
-    for (int64_t u = u0 + n_groups * kGroup + tid; u < u1; u += kRowWG) consume(p[u], u);
+    for (int64_t u = u0 + n_groups * kGroup + tid; u < u1; u += kRowWG) consume(__builtin_nontemporal_load(p + u), u);
     if (tid == 0) {
       for (int e = 0; e < n_tail; ++e) {
         float x[1] = {Elem<T>::load1(row + n_units * kVec + e)};
@@ -656,13 +656,13 @@ int row_splits_for(int64_t rows, int64_t V, int vec);
 // splits 23 us, 32 splits 27 us, 12 splits 37 us; 256 rows: 20 splits 47 us, the row kernel's 8 splits
 // 68 us).  Very small batches still get enough workgroups to pull a row from many CUs.  Larger batches follow the
 // row kernel (one workgroup per row from 512 rows on, which streams the row once); where that takes over was measured
-// at V = 151936, ranges against the row kernel's policy: fp32 512 / 768 / 1024 / 1280 rows 63.9 / 89.4 / 116.3 / 145.1 us
-// against 85.0 / 97.4 / 118.8 / 143.8; bf16 300 / 350 / 400 / 512 rows 46.7 / 51.6 / 56.9 / 69.1 against 51.5 / 52.0 /
-// 54.6 / 61.5 (a bf16 range holds twice the elements per byte, and it is the per-element work that costs).
+// at V = 151936, ranges against the row kernel's policy: fp32 512 / 768 / 900 / 1024 / 1152 rows 62.5 / 85.4 / 97.4 / 110.5 /
+// 125.2 us against 83.0 / 92.6 / 100.5 / 107.9 / 121.4; bf16 256 / 300 / 340 / 400 rows 41.3 / 46.6 / 50.5 / 56.8 against 47.7 /
+// 50.4 / 50.9 / 53.6 (a bf16 range holds twice the elements per byte, and it is the per-element work that costs).
 static int sample_splits_for(int64_t rows, int64_t V, int vec) {
   const int base = row_splits_for(rows, V, vec);
   int64_t s = (V + 8191) / 8192;
-  const int64_t most_ranges = vec == 4 ? 20000 : 6500;   // rows * ranges: ~1050 fp32 rows, ~340 bf16 rows at V = 151936
+  const int64_t most_ranges = vec == 4 ? 18000 : 6500;   // rows * ranges: ~950 fp32 rows, ~340 bf16 rows at V = 151936
   if (rows * s > most_ranges) return base;
   const int64_t fill = (512 + rows - 1) / rows;
   if (s < fill) s = fill;
