@@ -1223,11 +1223,28 @@ __device__ __forceinline__ void combine_one(const FusedPartial* parts, int n_par
                                             RowStat& st, float& tx) {
   st = stat_identity();
   tx = -INFINITY;
-  for (int q = lane; q < n_parts; q += 64) {
-    const FusedPartial p = parts[q];
-    RowStat o{p.mx, p.s, p.w, p.bi};
-    stat_merge(st, o, scale);
-    tx = fmaxf(tx, p.tx);
+  // A lane's partials are fetched eight at a time before the first is merged (clamped, unconditional loads: all in
+  // flight together): the merges form a chain, and a load inside it costs a trip to memory per partial - the previous
+  // launch wrote these records on other dies.  Same merge order as a plain loop.
+  constexpr int kBatch = 8;
+  for (int base = 0; base < n_parts; base += 64 * kBatch) {
+    f32x4 head[kBatch];
+    int bi[kBatch];
+#pragma unroll
+    for (int q = 0; q < kBatch; ++q) {
+      const int i = base + lane + 64 * q;
+      const FusedPartial* src = parts + (i < n_parts ? i : n_parts - 1);
+      head[q] = *reinterpret_cast<const f32x4*>(src);  // mx, s, w, tx
+      bi[q] = src->bi;
+    }
+#pragma unroll
+    for (int q = 0; q < kBatch; ++q) {
+      if (base + lane + 64 * q < n_parts) {
+        RowStat o{head[q][0], head[q][1], head[q][2], bi[q]};
+        stat_merge(st, o, scale);
+        tx = fmaxf(tx, head[q][3]);
+      }
+    }
   }
   stat_wave_reduce(st, scale);
 #pragma unroll
@@ -1365,10 +1382,10 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   // The third W buffer (see the kernel), measured against the two-buffer form in the same runs.  One or two token tiles:
   // 6-13 % faster with any outputs (256 x 1024: 96 -> 87 us, 256 x 4096: 338 -> 297, 512 x 4096: 534 -> 503).  More token
   // tiles, log-probs only: 4096 x 1024 -2.3 %, 8192 x 1024 -1.5 %, 1024 x 4096 -5 %, 4096 x 4096 -1.7 %, 16384 x 2560 -2.6 %,
-  // but 8192 x 4096 +0.2 %, 32768 x 4096 +0.7 %, 65536 x 4096 +0.5..2 %.  With the entropy or the argmax the epilogue of
+  // 8192 x 4096 -1.6..+0.2 % over boxes, but 32768 x 4096 +0.7 %, 65536 x 4096 +0.5..2 %.  With the entropy or the argmax the epilogue of
   // the deeper form spills 15-37 registers around every fold and it is 2.5 % slower at 4096 x 1024, equal at K = 4096.
   p.dma_deep = 0;
-  if (p.dma_nbt == 4) p.dma_deep = n_tokens <= 512 ? 2 : ((H < 4096 || n_tokens < 8192) ? 1 : 0);
+  if (p.dma_nbt == 4) p.dma_deep = n_tokens <= 512 ? 2 : ((H < 4096 || n_tokens <= 8192) ? 1 : 0);
   p.unit32 = 8;   // 32-row blocks per vocab unit: whole 256-row tiles unless the DMA kernel is given something finer below
   if (H % k2BK == 0) p.kind = kDma;
   // The streaming kernel runs one workgroup per CU: without a CU count (no device) the tiled kernels serve.
