@@ -111,13 +111,17 @@ struct RowStat {
 __device__ __forceinline__ RowStat stat_identity() { return RowStat{kMaxFloor, 0.f, 0.f, 0x7fffffff}; }
 
 // Merge b into a.  Ties on mx keep the lower unit index, so the first maximum wins.
+// w = sum (y - m) 2^(y - m) is taken RELATIVE to the state's own maximum (y = x * scale, m = mx * scale; every term <= 0):
+// moving a state to a larger maximum m' turns it into 2^(m - m') * (w + (m - m') * s).  The entropy then needs no m at
+// all - ln 2 * (log2 s - w / s) - where sum y 2^(y - m) would have it cancel against m + log2 s at the logits' magnitude.
 __device__ __forceinline__ void stat_merge(RowStat& a, const RowStat& b, float scale) {
   const float mx = fmaxf(a.mx, b.mx);
-  const float fa = fast_exp2((a.mx - mx) * scale);
-  const float fb = fast_exp2((b.mx - mx) * scale);
+  const float da = (a.mx - mx) * scale, db = (b.mx - mx) * scale;  // finite: the maxima start at kMaxFloor, not at -inf
+  const float fa = fast_exp2(da);
+  const float fb = fast_exp2(db);
   const int bi = (b.mx > a.mx || (b.mx == a.mx && b.bi < a.bi)) ? b.bi : a.bi;
+  a.w = fmaf(da, a.s, a.w) * fa + fmaf(db, b.s, b.w) * fb;
   a.s = a.s * fa + b.s * fb;
-  a.w = a.w * fa + b.w * fb;
   a.mx = mx;
   a.bi = bi;
 }

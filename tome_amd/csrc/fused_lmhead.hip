@@ -236,21 +236,24 @@ __device__ __forceinline__ void fold_tile(f32x16 (&acc)[NBV][NBT], RowStat (&st)
         cm = raw_max(cm, m);
       }
     }
-    const float resc = fast_exp2((st[j].mx - cm) * scale);
+    const float dm = (st[j].mx - cm) * scale;
+    const float resc = fast_exp2(dm);
     const float m = cm * scale;
-    float s0 = st[j].s * resc, s1 = 0.f, w0 = ENT ? st[j].w * resc : 0.f, w1 = 0.f;
+    // w: sum (y - m) 2^(y - m), relative to the running maximum (stat_merge has the rule for moving it)
+    float s0 = st[j].s * resc, s1 = 0.f, w0 = ENT ? fmaf(dm, st[j].s, st[j].w) * resc : 0.f, w1 = 0.f;
 #pragma unroll
     for (int i = 0; i < NBV; ++i)
 #pragma unroll
       for (int e = 0; e < 16; e += 2) {
         const float x0 = acc[i][j][e], x1 = acc[i][j][e + 1];
-        const float e0 = fast_exp2(fmaf(x0, scale, -m));
-        const float e1 = fast_exp2(fmaf(x1, scale, -m));
+        const float t0 = fmaf(x0, scale, -m), t1 = fmaf(x1, scale, -m);
+        const float e0 = fast_exp2(t0);
+        const float e1 = fast_exp2(t1);
         s0 += e0;
         s1 += e1;
-        if constexpr (ENT) {
-          w0 = fmaf(clamp_below(x0) * scale, e0, w0);
-          w1 = fmaf(clamp_below(x1) * scale, e1, w1);
+        if constexpr (ENT) {  // a masked row (-inf): floor * 0, not -inf * 0
+          w0 = fmaf(clamp_below(t0), e0, w0);
+          w1 = fmaf(clamp_below(t1), e1, w1);
         }
       }
     st[j].mx = cm;
@@ -457,21 +460,24 @@ __device__ __forceinline__ void fold_tile16(f32x4v (&acc)[NBV_ALLOC][NBT], RowSt
         cm = raw_max(cm, bm);
       }
     }
-    const float resc = fast_exp2((st[j].mx - cm) * scale);
+    const float dm = (st[j].mx - cm) * scale;
+    const float resc = fast_exp2(dm);
     const float m = cm * scale;
-    float s0 = st[j].s * resc, s1 = 0.f, w0 = ENT ? st[j].w * resc : 0.f, w1 = 0.f;
+    // w: sum (y - m) 2^(y - m), relative to the running maximum (stat_merge has the rule for moving it)
+    float s0 = st[j].s * resc, s1 = 0.f, w0 = ENT ? fmaf(dm, st[j].s, st[j].w) * resc : 0.f, w1 = 0.f;
 #pragma unroll
     for (int i = 0; i < NBV; ++i)
 #pragma unroll
       for (int e = 0; e < 4; e += 2) {
         const float x0 = acc[i][j][e], x1 = acc[i][j][e + 1];
-        const float e0 = fast_exp2(fmaf(x0, scale, -m));
-        const float e1 = fast_exp2(fmaf(x1, scale, -m));
+        const float t0 = fmaf(x0, scale, -m), t1 = fmaf(x1, scale, -m);
+        const float e0 = fast_exp2(t0);
+        const float e1 = fast_exp2(t1);
         s0 += e0;
         s1 += e1;
-        if constexpr (ENT) {
-          w0 = fmaf(clamp_below(x0) * scale, e0, w0);
-          w1 = fmaf(clamp_below(x1) * scale, e1, w1);
+        if constexpr (ENT) {  // a masked row (-inf): floor * 0, not -inf * 0
+          w0 = fmaf(clamp_below(t0), e0, w0);
+          w1 = fmaf(clamp_below(t1), e1, w1);
         }
       }
     st[j].mx = cm;
@@ -1279,7 +1285,7 @@ __global__ __launch_bounds__(256) void fused_combine_kernel(CombineArgs a) {
   if (a.out_argmax) a.out_argmax[tok] = st.bi == 0x7fffffff ? 0 : st.bi;
   if (a.out_lp) a.out_lp[tok] = lp;
   if (a.out_lse) a.out_lse[tok] = (m + log2s) * kLn2;
-  if (a.out_entropy) a.out_entropy[tok] = (m + log2s - st.w / st.s) * kLn2;
+  if (a.out_entropy) a.out_entropy[tok] = (log2s - st.w / st.s) * kLn2;
   if (a.out_ref_lp) a.out_ref_lp[tok] = ref_lp;
   if (a.out_k3) {
     const float d = ref_lp - lp;

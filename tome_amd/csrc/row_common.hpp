@@ -56,15 +56,17 @@ __device__ __forceinline__ float absorb(RowStat& st, const float (&x)[N], int un
   const float cm = max_of<N>(x);
   const float mx_new = fmaxf(st.mx, cm);
   if constexpr (AMAX) st.bi = (cm > st.mx) ? unit : st.bi;
-  const float resc = fast_exp2((st.mx - mx_new) * scale);
+  const float d = (st.mx - mx_new) * scale;
+  const float resc = fast_exp2(d);
   const float m = mx_new * scale;
+  float w = ENT ? fmaf(d, st.s, st.w) * resc : 0.f;  // relative to the new maximum (see stat_merge)
   float s = st.s * resc;
-  float w = ENT ? st.w * resc : 0.f;
 #pragma unroll
   for (int i = 0; i < N; ++i) {
-    const float e = fast_exp2(fmaf(x[i], scale, -m));
+    const float t = fmaf(x[i], scale, -m);
+    const float e = fast_exp2(t);
     s += e;
-    if constexpr (ENT) w = fmaf(fmaxf(x[i], kMaxFloor) * scale, e, w);
+    if constexpr (ENT) w = fmaf(clamp_below(t), e, w);  // a -inf logit: floor * 0, not -inf * 0
   }
   st.mx = mx_new;
   st.s = s;

@@ -70,7 +70,7 @@ __device__ __forceinline__ void finish_row(const RowArgs& a, const T* row, int64
   const float log2s = fast_log2(st.s);
   if (a.out_lp) a.out_lp[r] = (fmaf(x_t, a.scale, -m) - log2s) * kLn2;  // NaN in, NaN out
   if (a.out_lse) a.out_lse[r] = (m + log2s) * kLn2;
-  if constexpr (ENT) a.out_entropy[r] = (m + log2s - st.w / st.s) * kLn2;
+  if constexpr (ENT) a.out_entropy[r] = (log2s - st.w / st.s) * kLn2;  // w is relative to the maximum: no m here
   if constexpr (AMAX) a.out_argmax[r] = argmax_in_unit<T, true>(row, a.V, st.bi, st.mx);
 }
 
