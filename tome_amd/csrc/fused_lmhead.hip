@@ -1310,7 +1310,7 @@ struct FusedPlan {
   FusedKind kind;
   int dma_nbt;                               // kDma only: token blocks per wave (4, 2 or 1: 256, 128 or 64 tokens per tile)
   int unit32;                                // kDma only: 32-row blocks per vocab unit (1 = mixed tile heights; 7 / 8 = whole tiles of 224 / 256 rows)
-  int dma_deep;                              // kDma, 256-token tile only: three W buffers - 0 never, 1 for sweeps without entropy and argmax, 2 always
+  int dma_deep;                              // kDma, 256-token tile only: three W buffers - 0 never, 1 for sweeps without the entropy, 2 always
   int small_nbt, small_ksteps, small_waves;  // kSmall only
   int bt, slots;
   int n_vunits, upt;   // vocab units the splits share out, and units per 256-row tile (what a unit costs, for the schedule)
@@ -1388,10 +1388,11 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   // The third W buffer (see the kernel), measured against the two-buffer form in the same runs.  One or two token tiles:
   // 6-13 % faster with any outputs (256 x 1024: 96 -> 87 us, 256 x 4096: 338 -> 297, 512 x 4096: 534 -> 503).  More token
   // tiles, log-probs only: 4096 x 1024 -2.3 %, 8192 x 1024 -1.5 %, 1024 x 4096 -5 %, 4096 x 4096 -1.7 %, 16384 x 2560 -2.6 %,
-  // 8192 x 4096 -1.6..+0.2 % over boxes, but 32768 x 4096 +0.7 %, 65536 x 4096 +0.5..2 %.  With the entropy or the argmax the epilogue of
-  // the deeper form spills 15-37 registers around every fold and it is 2.5 % slower at 4096 x 1024, equal at K = 4096.
+  // 8192 x 4096 -1.6..+0.2 % over boxes, but 32768 x 4096 +0.7 %, 65536 x 4096 +0.5..2 %.  With the argmax alone it follows
+  // (1024 x 4096 -4 %, 4096 x 1024 equal, 8192 x 4096 -1 %); with the entropy the fold of the deeper form spills 29-37
+  // registers around every tile change: 1024 x 4096 -3 %, but 4096 x 1024 +2.6 % and 8192 x 4096 +2.3 %.
   p.dma_deep = 0;
-  if (p.dma_nbt == 4) p.dma_deep = n_tokens <= 512 ? 2 : ((H < 4096 || n_tokens <= 8192) ? 1 : 0);
+  if (p.dma_nbt == 4) p.dma_deep = n_tokens <= 1024 ? 2 : ((H < 4096 || n_tokens <= 8192) ? 1 : 0);
   p.unit32 = 8;   // 32-row blocks per vocab unit: whole 256-row tiles unless the DMA kernel is given something finer below
   if (H % k2BK == 0) p.kind = kDma;
   // The streaming kernel runs one workgroup per CU: without a CU count (no device) the tiled kernels serve.
@@ -1533,7 +1534,7 @@ static int launch_main(const FusedArgs& a, const FusedPlan& plan, bool want_argm
     return n;  // >= 2: fused_plan only picks this kernel when it can be placed
   }
   if (plan.kind == kDma) {
-    if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.unit32, plan.dma_deep == 2, plan.grid, stream);
+    if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.unit32, plan.dma_deep >= (ENT ? 2 : 1), plan.grid, stream);
     else launch_dma<ENT, false>(a, plan.dma_nbt, plan.unit32, plan.dma_deep >= (ENT ? 2 : 1), plan.grid, stream);
   } else {
     if (want_argmax) hipLaunchKernelGGL((fused_lmhead_kernel<ENT, true>), dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
