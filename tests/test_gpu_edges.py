@@ -133,10 +133,9 @@ def test_row_extreme_temperature(dev, dtype, T, rows, V):
 # ---- fused kernels ------------------------------------------------------------------------------------
 # (kernel, n, H, V): the streaming kernel takes <= 64 tokens with H % 256 == 0, the LDS-DMA kernel H % 64 == 0
 # (forced for the batch sizes used here as well: 100 and 300 tokens run its 128-token tile, 200 tokens one 256-token tile on
-# three W buffers, 600 tokens three 256-token tiles on two - with the entropy and the argmax asked for), the generic kernel
-# everything else.
+# three W buffers, 1100 tokens five 256-token tiles on two - with the entropy asked for), the generic kernel everything else.
 FUSED = [("small", 48, 1024, 3000), ("dma", 300, 256, 3000), ("dma", 100, 256, 3000), ("dma", 200, 256, 3000),
-         ("dma", 600, 256, 3000), ("generic", 150, 72, 3000)]
+         ("dma", 1100, 128, 3000), ("generic", 150, 72, 3000)]
 
 
 @pytest.fixture
