@@ -31,6 +31,8 @@ def _safe_uniforms(x64, T, k, rng):
     (64, V_QWEN3, torch.float32, 1.0, 20), (32, V_QWEN3, torch.bfloat16, 0.7, 20), (7, 4099, torch.float32, 1.3, 20),
     (5, 2048, torch.float32, 1.0, 5), (9, 2049, torch.bfloat16, 0.5, 32), (3, 17, torch.float32, 1.0, 20),
     (4, 300, torch.bfloat16, 2.0, 1), (130, 8191, torch.float32, 0.9, 20),
+    # 512 rows and more: still cut into ranges of 8192 elements (fp32, and bf16 while the batch is small) ...
+    (600, 30000, torch.float32, 1.0, 20), (700, 40000, torch.bfloat16, 0.8, 20),
 ])
 def test_sampler_matches_oracle(dev, rows, V, dtype, T, k):
     rng = np.random.default_rng(rows * 31 + V)
@@ -47,6 +49,28 @@ def test_sampler_matches_oracle(dev, rows, V, dtype, T, k):
     np.testing.assert_array_equal(got.argmax.cpu().numpy(), np.argmax(x64, axis=-1))
     # the same pass must agree with the plain row kernel on the drawn ids
     lp2 = tome_amd.token_logprobs(x, got.token, T).lp
+    np.testing.assert_allclose(got.lp.cpu().numpy(), lp2.cpu().numpy(), atol=2e-6, rtol=0)
+
+
+@pytest.mark.parametrize("rows,V,dtype", [(2300, 65536, torch.float32), (1700, 32768, torch.bfloat16)])
+def test_sampler_streams_large_batches(dev, rows, V, dtype):
+    """Batches beyond ~950 fp32 / ~340 bf16 rows of 151936 (counted in ranges of 8192 elements) take one streaming
+    workgroup per row; at that size the check runs on the GPU: the candidates' logits against torch.topk (values: ids
+    may differ among equal logits), the greedy id against torch.argmax wherever the maximum is unique, the log-prob of
+    the drawn id against the row kernel."""
+    k = 20
+    g = torch.Generator(device=dev).manual_seed(5)
+    x = (torch.randn((rows, V), device=dev, generator=g) * 2.0).to(dtype)
+    u = torch.rand(rows, device=dev, generator=g)
+    got = tome_amd.sample_tokens(x, 1.1, k, uniforms=u, want_topk=True)
+    vals, _ = torch.topk(x.float(), k, dim=-1)
+    assert torch.equal(got.topk_logit, vals)
+    assert torch.equal(x.float().gather(1, got.topk_idx.long()), vals)
+    unique = vals[:, 0] > vals[:, 1]
+    assert torch.equal(got.argmax[unique].long(), torch.argmax(x.float(), dim=-1)[unique])
+    in_topk = (got.topk_idx == got.token[:, None]).any(dim=1)
+    assert bool(in_topk.all())
+    lp2 = tome_amd.token_logprobs(x, got.token, 1.1).lp
     np.testing.assert_allclose(got.lp.cpu().numpy(), lp2.cpu().numpy(), atol=2e-6, rtol=0)
 
 
