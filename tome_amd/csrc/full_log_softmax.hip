@@ -119,9 +119,11 @@ __global__ __launch_bounds__(kFullWG) void full_log_softmax_kernel(FullArgs a) {
 }
 
 // ---- one pass for bf16 rows that fit a workgroup's registers ----------------------------------------
-// A 1024-lane workgroup (one per CU) loads a whole row - up to CH 16-byte units per lane, all in flight together -
-// takes the row's maximum and sum from the registers (two sweeps, as the sampler's cached variant does) and writes
-// T(x * inv_temp) - T(lse) from the same registers: the matrix is read ONCE and written once.
+// A 1024-lane workgroup (one per CU) holds a whole row in registers - up to CH 16-byte units per lane, all requested
+// together - and writes T(x * inv_temp) - T(lse) from the same registers: the matrix is read ONCE and written once.
+// With a single workgroup on the CU nothing else covers its arithmetic, so every lane keeps a running (maximum, sum) of
+// its own and takes in each unit as it arrives (the row kernel's online update) instead of a sweep for the maximum, a
+// barrier and a sweep for the sum after the last byte has landed; the lanes' states are merged through one barrier.
 template <int CH>
 __global__ __launch_bounds__(1024) void full_log_softmax_onepass_kernel(FullArgs a) {
   constexpr int kWaves = 16;
@@ -134,95 +136,109 @@ __global__ __launch_bounds__(1024) void full_log_softmax_onepass_kernel(FullArgs
   u32x4* dst = reinterpret_cast<u32x4*>(out_row);
   const int n_units = (int)(a.V / 8);
   const int n_tail = (int)(a.V - (int64_t)n_units * 8);  // single elements after the last whole unit: lane 0
+  const float scale = a.scale;
   u32x4 v[CH];
 #pragma unroll
   for (int q = 0; q < CH; ++q) {  // unconditional (clamped) loads; unit 0 exists (checked on the host)
     const int u = tid + q * 1024;
     v[q] = __builtin_nontemporal_load(src + (u < n_units ? u : 0));
   }
-  float tail[7];
-#pragma unroll
-  for (int e = 0; e < 7; ++e) tail[e] = (tid == 0 && e < n_tail) ? bf16_bits_to_f32(in_row[(int64_t)n_units * 8 + e]) : -INFINITY;
-  float m = -INFINITY;
+  // the lane's running maximum (floored like every kernel of this path) and sum of 2^((x - maximum) * scale)
+  float lm = kMaxFloor, ls = 0.f;
 #pragma unroll
   for (int q = 0; q < CH; ++q)
     if (tid + q * 1024 < n_units) {
       float x[8];
       Elem<uint16_t>::unpack(v[q], x);
-      m = fmaxf(m, max_of<8>(x));
-    }
+      const float nm = raw_max3(raw_max3(x[0], x[1], x[2]), raw_max3(x[3], x[4], x[5]), raw_max3(lm, x[6], x[7]));
+      const float m = nm * scale;
+      float s0 = ls * fast_exp2((lm - nm) * scale), s1 = 0.f;
 #pragma unroll
-  for (int e = 0; e < 7; ++e) m = fmaxf(m, tail[e]);
-  m = fmaxf(m, wave_exchange<0>(m));
-  m = fmaxf(m, wave_exchange<1>(m));
-  m = fmaxf(m, wave_exchange<2>(m));
-  m = fmaxf(m, wave_exchange<3>(m));
-  m = fmaxf(m, wave_exchange<4>(m));
-  m = fmaxf(m, wave_exchange<5>(m));
-  if (lane == 0) red_m[wave] = m;
+      for (int i = 0; i < 8; i += 2) {
+        s0 += fast_exp2(fmaf(x[i], scale, -m));
+        s1 += fast_exp2(fmaf(x[i + 1], scale, -m));
+      }
+      ls = s0 + s1;
+      lm = nm;
+    }
+  if (n_tail != 0 && tid == 0) {  // rare (V not a multiple of 8): fetched here, so that no wait stands in front of the sweep
+    for (int e = 0; e < n_tail; ++e) {
+      const float x = bf16_bits_to_f32(in_row[(int64_t)n_units * 8 + e]);
+      const float nm = fmaxf(lm, x);
+      ls = ls * fast_exp2((lm - nm) * scale) + fast_exp2(fmaf(x, scale, -nm * scale));
+      lm = nm;
+    }
+  }
+  auto merge = [&](float om, float os) {
+    const float nm = fmaxf(lm, om);
+    ls = ls * fast_exp2((lm - nm) * scale) + os * fast_exp2((om - nm) * scale);
+    lm = nm;
+  };
+  merge(wave_exchange<0>(lm), wave_exchange<0>(ls));
+  merge(wave_exchange<1>(lm), wave_exchange<1>(ls));
+  merge(wave_exchange<2>(lm), wave_exchange<2>(ls));
+  merge(wave_exchange<3>(lm), wave_exchange<3>(ls));
+  merge(wave_exchange<4>(lm), wave_exchange<4>(ls));
+  merge(wave_exchange<5>(lm), wave_exchange<5>(ls));
+  if (lane == 0) {
+    red_m[wave] = lm;
+    red_s[wave] = ls;
+  }
   __syncthreads();
   float mx = red_m[0];
 #pragma unroll
   for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, red_m[w]);
-  mx = fmaxf(mx, kMaxFloor);  // the floor of the running maximum that every kernel of this path shares
-  const float mm = mx * a.scale;
-  float s0 = 0.f, s1 = 0.f;
-#pragma unroll
-  for (int q = 0; q < CH; ++q)
-    if (tid + q * 1024 < n_units) {
-      float x[8];
-      Elem<uint16_t>::unpack(v[q], x);
-#pragma unroll
-      for (int i = 0; i < 8; i += 2) {
-        s0 += fast_exp2(fmaf(x[i], a.scale, -mm));
-        s1 += fast_exp2(fmaf(x[i + 1], a.scale, -mm));
-      }
-    }
-#pragma unroll
-  for (int e = 0; e < 7; ++e) s0 += fast_exp2(fmaf(tail[e], a.scale, -mm));  // -inf adds nothing
-  float ws = s0 + s1;
-  ws += wave_exchange<0>(ws);
-  ws += wave_exchange<1>(ws);
-  ws += wave_exchange<2>(ws);
-  ws += wave_exchange<3>(ws);
-  ws += wave_exchange<4>(ws);
-  ws += wave_exchange<5>(ws);
-  if (lane == 0) red_s[wave] = ws;
-  __syncthreads();
   float sum = 0.f;
 #pragma unroll
-  for (int w = 0; w < kWaves; ++w) sum += red_s[w];
-  const float lse = (mm + fast_log2(sum)) * kLn2;
+  for (int w = 0; w < kWaves; ++w) sum += red_s[w] * fast_exp2((red_m[w] - mx) * scale);
+  const float lse = (mx * scale + fast_log2(sum)) * kLn2;
   if (tid == 0) a.row_lse[r] = lse;
   const float lse_t = bf16_rt(lse);
+  if (a.inv_temp == 1.0f) {  // the usual call: T(x * 1) is x itself, one rounding and two operations per pair fewer
 #pragma unroll
-  for (int q = 0; q < CH; ++q) {
-    const int u = tid + q * 1024;
-    if (u < n_units) {
-      u32x4 o;
-      o.x = sub_pack_bf16(v[q].x, a.inv_temp, lse_t);
-      o.y = sub_pack_bf16(v[q].y, a.inv_temp, lse_t);
-      o.z = sub_pack_bf16(v[q].z, a.inv_temp, lse_t);
-      o.w = sub_pack_bf16(v[q].w, a.inv_temp, lse_t);
-      __builtin_nontemporal_store(o, dst + u);
+    for (int q = 0; q < CH; ++q) {
+      const int u = tid + q * 1024;
+      if (u < n_units) {
+        u32x4 o;
+        o.x = pack_bf16(__fsub_rn(bf16_lo(v[q].x), lse_t), __fsub_rn(bf16_hi(v[q].x), lse_t));
+        o.y = pack_bf16(__fsub_rn(bf16_lo(v[q].y), lse_t), __fsub_rn(bf16_hi(v[q].y), lse_t));
+        o.z = pack_bf16(__fsub_rn(bf16_lo(v[q].z), lse_t), __fsub_rn(bf16_hi(v[q].z), lse_t));
+        o.w = pack_bf16(__fsub_rn(bf16_lo(v[q].w), lse_t), __fsub_rn(bf16_hi(v[q].w), lse_t));
+        __builtin_nontemporal_store(o, dst + u);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < CH; ++q) {
+      const int u = tid + q * 1024;
+      if (u < n_units) {
+        u32x4 o;
+        o.x = sub_pack_bf16(v[q].x, a.inv_temp, lse_t);
+        o.y = sub_pack_bf16(v[q].y, a.inv_temp, lse_t);
+        o.z = sub_pack_bf16(v[q].z, a.inv_temp, lse_t);
+        o.w = sub_pack_bf16(v[q].w, a.inv_temp, lse_t);
+        __builtin_nontemporal_store(o, dst + u);
+      }
     }
   }
-  if (tid == 0)
-    for (int e = 0; e < n_tail; ++e)
-      out_row[(int64_t)n_units * 8 + e] = f32_to_bf16_bits(__fsub_rn(bf16_rt(__fmul_rn(tail[e], a.inv_temp)), lse_t));
+  if (n_tail != 0 && tid == 0)
+    for (int e = 0; e < n_tail; ++e) {
+      const float x = bf16_bits_to_f32(in_row[(int64_t)n_units * 8 + e]);
+      out_row[(int64_t)n_units * 8 + e] = f32_to_bf16_bits(__fsub_rn(bf16_rt(__fmul_rn(x, a.inv_temp)), lse_t));
+    }
 }
 
 constexpr int kOnePassUnits = 19;  // 16-byte units per lane: 1024 lanes hold 155648 bf16 elements
 
 // Whether the one-pass kernel takes this call: bf16, 16-byte aligned rows, a row that fits the registers of one
 // workgroup and is long enough to keep most of its 1024 lanes busy.
-// One workgroup per row leaves most of the chip idle on a decode-sized batch: below ~96 rows the two-pass kernels, which
-// split a row over several workgroups, are faster (8 / 32 / 64 rows of 151936 bf16: 7.9 / 11.6 / 16.5 us against 17.3 /
-// 18.0 / 18.5; 128 / 512 / 2048 rows: 25.4 / 77.5 / 291 against 20.1 / 63.6 / 238).
+// One workgroup per row leaves most of the chip idle on a decode-sized batch: below ~44 rows the two-pass kernels, which
+// split a row over several workgroups, are faster (8 / 32 / 48 / 64 / 80 rows of 151936 bf16: 8.1 / 11.6 / 14.3 / 16.5 /
+// 19.4 us against 12.8 / 13.2 / 13.3 / 13.4 / 13.7; 128 / 512 / 2048 rows: 25.4 / 77.5 / 291 against 16.9 / 58.4 / 227).
 bool full_log_softmax_one_pass(const void* in, const void* out, int dtype, int64_t rows, int64_t V, int64_t in_stride, int64_t out_stride) {
   const bool aligned = reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
                        in_stride % 8 == 0 && out_stride % 8 == 0;
-  return dtype == 1 && aligned && rows >= 96 && V >= 16384 && V / 8 <= (int64_t)kOnePassUnits * 1024;
+  return dtype == 1 && aligned && rows >= 44 && V >= 16384 && V / 8 <= (int64_t)kOnePassUnits * 1024;
 }
 
 hipError_t full_log_softmax_onepass_launch(const void* in, void* out, int64_t rows, int64_t V, int64_t in_stride,

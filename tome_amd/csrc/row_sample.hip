@@ -330,7 +330,7 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
       if (u0 + tid + q * kRowWG < u1) {
         float x[kVec];
         Elem<T>::unpack(cached[q], x);
-        lane_max = fmaxf(lane_max, max_of<kVec>(x));
+        lane_max = fmaxf(lane_max, max_of_raw<kVec>(x));
       }
 #pragma unroll
     for (int e = 0; e < kVec - 1; ++e) lane_max = fmaxf(lane_max, tail[e]);
@@ -412,7 +412,7 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
       for (int q = 0; q < kRowUnroll; ++q) {
         float x[kVec];
         Elem<T>::unpack(first[q], x);
-        if (max_of<kVec>(x) >= early_val) {
+        if (max_of_raw<kVec>(x) >= early_val) {
 #pragma unroll
           for (int i = 0; i < kVec; ++i) offer(x[i], (u0 + tid + q * kRowWG) * kVec + i, early, early_val);
         }
@@ -483,7 +483,7 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
         if (u0 + tid + q * kRowWG < u1) {
           float x[kVec];
           Elem<T>::unpack(cached[q], x);
-          if (max_of<kVec>(x) >= theta_val) {
+          if (max_of_raw<kVec>(x) >= theta_val) {
 #pragma unroll
             for (int i = 0; i < kVec; ++i) offer(x[i], first_elem + (uint32_t)(q * kRowWG * kVec + i), theta, theta_val);
           }
@@ -528,7 +528,7 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
           for (int q = 0; q < kRowUnroll; ++q) {
             float x[kVec];
             Elem<T>::unpack(v[q], x);
-            if (max_of<kVec>(x) >= theta_val) {
+            if (max_of_raw<kVec>(x) >= theta_val) {
 #pragma unroll
               for (int i = 0; i < kVec; ++i) offer2(x[i], (u + q * kRowWG) * kVec + i);
             }
@@ -537,7 +537,7 @@ __global__ __launch_bounds__(kRowWG) __attribute__((amdgpu_waves_per_eu(6, 8))) 
         for (; u < u1; u += kRowWG) {
           float x[kVec];
           Elem<T>::unpack(p[u], x);
-          if (max_of<kVec>(x) >= theta_val) {
+          if (max_of_raw<kVec>(x) >= theta_val) {
 #pragma unroll
             for (int i = 0; i < kVec; ++i) offer2(x[i], u * kVec + i);
           }
