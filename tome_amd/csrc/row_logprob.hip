@@ -74,7 +74,9 @@ __device__ __forceinline__ void finish_row(const RowArgs& a, const T* row, int64
   if constexpr (AMAX) a.out_argmax[r] = argmax_in_unit<T, true>(row, a.V, st.bi, st.mx);
 }
 
-template <typename T, bool VECTOR, bool ENT, bool AMAX>
+// KEEP: the caller reads the rows again right away (the second pass of the full log-softmax matrix), so they are
+// loaded with ordinary loads and stay in the caches; everyone else streams them past the caches.
+template <typename T, bool VECTOR, bool ENT, bool AMAX, bool KEEP = false>
 __global__ __launch_bounds__(kRowWG) void row_logprob_kernel(RowArgs a) {
   constexpr int kVec = VECTOR ? Elem<T>::kVec : 1;
   __shared__ RowLds lds;
@@ -117,7 +119,7 @@ __global__ __launch_bounds__(kRowWG) void row_logprob_kernel(RowArgs a) {
     for (; u + (kRowUnroll - 1) * kRowWG < u1; u += kRowUnroll * kRowWG) {  // several 16-byte loads in flight per lane
       u32x4 v[kRowUnroll];
 #pragma unroll
-      for (int k = 0; k < kRowUnroll; ++k) v[k] = __builtin_nontemporal_load(p + u + k * kRowWG);
+      for (int k = 0; k < kRowUnroll; ++k) v[k] = KEEP ? p[u + k * kRowWG] : __builtin_nontemporal_load(p + u + k * kRowWG);
 #pragma unroll
       for (int k = 0; k < kRowUnroll; ++k) {
         float x[kVec];
@@ -129,7 +131,7 @@ __global__ __launch_bounds__(kRowWG) void row_logprob_kernel(RowArgs a) {
       u32x4 v[kRowUnroll - 1];
 #pragma unroll
       for (int k = 0; k < kRowUnroll - 1; ++k)
-        if (u + k * kRowWG < u1) v[k] = __builtin_nontemporal_load(p + u + k * kRowWG);
+        if (u + k * kRowWG < u1) v[k] = KEEP ? p[u + k * kRowWG] : __builtin_nontemporal_load(p + u + k * kRowWG);
 #pragma unroll
       for (int k = 0; k < kRowUnroll - 1; ++k)
         if (u + k * kRowWG < u1) {
@@ -197,9 +199,9 @@ __global__ __launch_bounds__(64) void row_combine_kernel(RowArgs a) {
   }
 }
 
-template <typename T, bool VECTOR, bool ENT, bool AMAX>
+template <typename T, bool VECTOR, bool ENT, bool AMAX, bool KEEP = false>
 static hipError_t launch_row(const RowArgs& a, int64_t rows, hipStream_t stream, bool skip_combine = false) {
-  hipLaunchKernelGGL((row_logprob_kernel<T, VECTOR, ENT, AMAX>), dim3((unsigned)(rows * a.splits)),
+  hipLaunchKernelGGL((row_logprob_kernel<T, VECTOR, ENT, AMAX, KEEP>), dim3((unsigned)(rows * a.splits)),
                      dim3(kRowWG), 0, stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || a.splits == 1 || skip_combine) return e;
@@ -282,10 +284,15 @@ hipError_t row_lse_partials_launch(const void* logits, int dtype, int64_t rows, 
   a.splits = row_splits_for(rows, V, vector_ok ? vec : 1);
   a.scale = kLog2e / temperature;
   *splits = a.splits;
+  // The caller's second pass reads the matrix again: up to ~3/4 GB it pays to leave the rows in the caches (measured, both
+  // passes, fp32 rows of 151936: 64 rows 25.9 -> 24.4 us, 512 rows 155 -> 145, 1024 rows 312 -> 294; 2048 rows 628 -> 648).
+  const bool keep = vector_ok && (double)rows * (double)V * esize <= 768.0 * 1024 * 1024;
   if (dtype == 0) {
+    if (keep) return launch_row<float, true, false, false, true>(a, rows, stream, true);
     return vector_ok ? launch_row<float, true, false, false>(a, rows, stream, true)
                      : launch_row<float, false, false, false>(a, rows, stream, true);
   }
+  if (keep) return launch_row<uint16_t, true, false, false, true>(a, rows, stream, true);
   return vector_ok ? launch_row<uint16_t, true, false, false>(a, rows, stream, true)
                    : launch_row<uint16_t, false, false, false>(a, rows, stream, true);
 }
