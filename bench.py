@@ -393,14 +393,15 @@ def bench_fused(dev, steps, warmup, n=4096, H=1024, temperature=1.0, lengths=Non
     return tm
 
 
-def bench_library_gemm(dev, steps, warmup, n=4096, H=1024):
-    """The vendor library's bf16 GEMM alone on config 3's shape, for scale: logits = hidden @ W^T written as bf16
-    [n, V] (what mlx-impl/model.py:538 materialises), no softmax.  torch.mm dispatches to hipBLASLt / rocBLAS."""
+def bench_library_gemm(dev, steps, warmup, n=4096, H=1024, vocab=V):
+    """The vendor library's bf16 GEMM alone, for scale: logits = hidden @ W^T written as bf16 [n, vocab] (what
+    mlx-impl/model.py:538 materialises), no softmax - on config 3's shape, and on a square 8192^3 product (the shape
+    such libraries are tuned for: what this part sustains on random operands).  torch.mm dispatches to hipBLASLt / rocBLAS."""
     import torch
     g = torch.Generator(device=dev).manual_seed(4321)
     hidden = torch.randn((n, H), device=dev, generator=g).to(torch.bfloat16)
-    weight = (torch.randn((V, H), device=dev, generator=g) * 0.02).to(torch.bfloat16)
-    out = torch.empty((n, V), device=dev, dtype=torch.bfloat16)
+    weight = (torch.randn((vocab, H), device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    out = torch.empty((n, vocab), device=dev, dtype=torch.bfloat16)
     wt = weight.t()
 
     def step():
@@ -408,7 +409,7 @@ def bench_library_gemm(dev, steps, warmup, n=4096, H=1024):
     step()
     torch.cuda.synchronize()
     tm = time_steps(step, steps, warmup, clock=True)
-    tm.update({"tokens": n, "H": H, "flop": 2.0 * n * H * V})
+    tm.update({"tokens": n, "H": H, "flop": 2.0 * n * H * vocab})
     return tm
 
 
@@ -1014,6 +1015,13 @@ def main():
                                    "[4096, 151936] written, no softmax", "tokens": t["tokens"], "hidden": t["H"], "vocab": V},
             "roofline": mfma_roofline(t["flop"], t["ms"], None, "vendor library GEMM (hipBLASLt / rocBLAS via torch.mm)", t.get("sclk_mhz"))}
         done("library_gemm_config3")
+        t = bench_library_gemm(dev, K, W, n=8192, H=8192, vocab=8192)
+        legs["library_gemm_square_8192"] = {
+            "value": t["flop"] / (t["ms"] * 1e-3) / 1e12, "unit": "TFLOP/s", **timing_fields(t), "dtype": "bf16 x bf16 -> bf16",
+            "config": {"workload": "for scale, not part of the path: torch.mm (vendor GEMM library) on 8192 x 8192 x 8192, random "
+                                   "operands", "m": 8192, "n": 8192, "k": 8192},
+            "roofline": mfma_roofline(t["flop"], t["ms"], None, "vendor library GEMM (hipBLASLt / rocBLAS via torch.mm)", t.get("sclk_mhz"))}
+        done("library_gemm_square_8192")
     if "config4" in only:
         t = bench_fused(dev, K, W, n=16 * 1024, H=2560, temperature=0.7, lengths=(16, 1024, 128, 1024), seed=444)
         legs["config4_fused_varlen"] = {
