@@ -144,9 +144,12 @@ def test_local_compute_logprobs_dropin(dev):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,V,T", [(1, V_QWEN3, 1.0), (3, 4096 * 2 + 1, 0.7), (64, 4096, 1.0), (5, 8192 + 384, 2.0)])
+@pytest.mark.parametrize("rows,V,T", [(1, V_QWEN3, 1.0), (3, 4096 * 2 + 1, 0.7), (64, 4096, 1.0), (5, 8192 + 384, 2.0),
+                                      (1400, 4100, 1.0), (1301, 1030, 0.7), (40, 2051, 1.3)])
 def test_fused_log_softmax_full_matrix(dev, dtype, rows, V, T):
-    """model.py:77-89 drop-in, incl. the kernel's tail cases (V % 4096 in {0, 1, 384})."""
+    """model.py:77-89 drop-in, incl. the kernel's tail cases (V % 4096 in {0, 1, 384}) and, for fp32, both sizes of the
+    second pass's workgroups (two loads per lane below 1300 rows, one from there on) with rows that end in a partial
+    workgroup and in single elements."""
     rng = np.random.default_rng(V + rows)
     x = torch.from_numpy(rng.standard_normal((rows, V)).astype(np.float32)).to(dev).to(dtype)
     out = tome_amd.fused_log_softmax(x, T)

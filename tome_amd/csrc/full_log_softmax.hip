@@ -39,7 +39,7 @@ __device__ __forceinline__ uint32_t sub_pack_bf16(uint32_t u, float inv_temp, fl
   return pack_bf16(__fsub_rn(bf16_lo(z), lse_t), __fsub_rn(bf16_hi(z), lse_t));
 }
 
-template <bool BF16, bool VECTOR>
+template <bool BF16, bool VECTOR, int UNROLL = kFullUnroll>
 __global__ __launch_bounds__(kFullWG) void full_log_softmax_kernel(FullArgs a) {
   const int64_t r = blockIdx.x / a.chunks;
   const int chunk = blockIdx.x % a.chunks;
@@ -103,14 +103,14 @@ __global__ __launch_bounds__(kFullWG) void full_log_softmax_kernel(FullArgs a) {
       return o;
     };
     int64_t u = u0 + threadIdx.x;
-    for (; u + (kFullUnroll - 1) * kFullWG < u1; u += kFullUnroll * kFullWG) {  // several 16-byte loads in flight per lane
-      u32x4 v[kFullUnroll];
+    for (; u + (UNROLL - 1) * kFullWG < u1; u += UNROLL * kFullWG) {  // several 16-byte loads in flight per lane
+      u32x4 v[UNROLL];
 #pragma unroll
-      for (int q = 0; q < kFullUnroll; ++q) v[q] = __builtin_nontemporal_load(src + u + q * kFullWG);
+      for (int q = 0; q < UNROLL; ++q) v[q] = __builtin_nontemporal_load(src + u + q * kFullWG);
 #pragma unroll
-      for (int q = 0; q < kFullUnroll; ++q) __builtin_nontemporal_store(convert(v[q]), dst + u + q * kFullWG);
+      for (int q = 0; q < UNROLL; ++q) __builtin_nontemporal_store(convert(v[q]), dst + u + q * kFullWG);
     }
-    for (; u < u1; u += kFullWG) __builtin_nontemporal_store(convert(src[u]), dst + u);
+    for (; u < u1; u += kFullWG) __builtin_nontemporal_store(convert(__builtin_nontemporal_load(src + u)), dst + u);
     if (chunk == a.chunks - 1 && threadIdx.x == 0)
       for (int64_t e = n_units * kVec; e < a.V; ++e) scalar_elem(e);
   } else {
@@ -281,18 +281,25 @@ hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t
   a.out_stride = out_stride;
   a.inv_temp = 1.0f / temperature;  // the reference multiplies by 1/temp (model.py:27)
   const int64_t units = V / (vector_ok ? vec : 1);
-  // Many short workgroups stream a read + write mix best (measured: aiming at 65536 workgroups instead of 4096
-  // takes 512 x 151936 fp32 from 165 to 150 us and 4096 x 151936 bf16 from 655 to 633 us, both passes included),
-  // as long as each still issues its four loads per lane.
+  // Many short workgroups stream a read + write mix best, as long as each still issues a few loads per lane.  bf16
+  // rows (a batch too small or rows too long for the one-pass kernel): four loads per lane and pass, aiming at 65536
+  // workgroups (against 4096: 4096 x 151936 bf16 655 -> 633 us, both passes included).  fp32 rows: workgroups of ONE pass
+  // of two loads per lane - of one load per lane from ~1300 rows on (both passes, rows of 151936 fp32, four / two / one load:
+  // 64 rows 24.4 / 24.2 / 26.6 us, 1024 rows 296 / 288 / 295, 2048 rows 629 / 618 / 588, 4096 rows 1370 / 1227 / 1168).
   int64_t chunks = (65536 + rows - 1) / rows;
-  const int64_t by_work = units / (kFullUnroll * kFullWG);
+  int64_t by_work = units / (kFullUnroll * kFullWG);
+  const int f32_unroll = rows >= 1300 ? 1 : 2;
+  if (dtype == 0 && vector_ok) {
+    chunks = by_work = units / (f32_unroll * kFullWG);
+  }
   if (chunks > by_work) chunks = by_work;
   if (chunks < 1) chunks = 1;
   a.chunks = (int)chunks;
   const dim3 grid((unsigned)(rows * chunks)), block(kFullWG);
   if (dtype == 0) {
-    if (vector_ok) hipLaunchKernelGGL((full_log_softmax_kernel<false, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((full_log_softmax_kernel<false, false>), grid, block, 0, stream, a);
+    if (!vector_ok) hipLaunchKernelGGL((full_log_softmax_kernel<false, false>), grid, block, 0, stream, a);
+    else if (f32_unroll == 1) hipLaunchKernelGGL((full_log_softmax_kernel<false, true, 1>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((full_log_softmax_kernel<false, true, 2>), grid, block, 0, stream, a);
   } else {
     if (vector_ok) hipLaunchKernelGGL((full_log_softmax_kernel<true, true>), grid, block, 0, stream, a);
     else hipLaunchKernelGGL((full_log_softmax_kernel<true, false>), grid, block, 0, stream, a);
