@@ -601,6 +601,11 @@ def bench_full_matrix(dev, steps, warmup, rows, dtype_name):
     passes = 2 if (dtype_name == "bf16" and V >= 16384 and V // 8 <= 19 * 1024) else 3
     tm.update({"rows": rows, "bytes": passes * rows * V * esize, "passes_over_the_matrix": passes,
                "bytes_if_three_passes": 3 * rows * V * esize})
+    if nbuf == 1:
+        # For scale: the same read + write volume through torch's elementwise kernel (tiny workgroups: the grain at which
+        # reads and writes mix best on this part), and torch's own log_softmax on the same matrix.
+        tm["torch_mul_same_bytes_ms"] = time_steps(lambda: torch.mul(xs[0], 2.0, out=outs[0]), steps, warmup)["ms"]
+        tm["torch_log_softmax_ms"] = time_steps(lambda: torch.log_softmax(xs[0], dim=-1), max(2, steps // 4), 1)["ms"]
     return tm
 
 
@@ -942,6 +947,7 @@ def main():
         for rows, dn in ((4096, "bf16"), (64, "f32")):
             t = bench_full_matrix(dev, K, W, rows, dn)
             shapes[f"{rows}x{V}_{dn}"] = {**timing_fields(t), "passes_over_the_matrix": t["passes_over_the_matrix"],
+                                          **{k: t[k] for k in ("torch_mul_same_bytes_ms", "torch_log_softmax_ms") if k in t},
                                           "gbs_if_priced_on_three_passes": t["bytes_if_three_passes"] / (t["ms"] * 1e-3) / 1e9,
                                           "roofline": hbm_roofline(
                 t["bytes"], t["ms"], traffic_of(f"full_log_softmax_{rows}rows_{dn}"),
