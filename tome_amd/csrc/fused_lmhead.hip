@@ -572,10 +572,13 @@ constexpr int dma_lds_bytes(int nbt, bool deep = false) {  // 131072 at nbt = 4,
   return dma_w_bufs(nbt, deep) * dma_w_bytes() + dma_bufs(nbt) * dma_h_bytes(nbt);
 }
 
-// Default cache policy: non-temporal requests for either operand measured 4-5 % slower.
+// AUX: the request's cache policy bits (0 = default, 2 = non-temporal).  Hidden rows always go with the default; W rows
+// do wherever several token tiles read them (there non-temporal requests for either operand measured 1.5-5 % slower),
+// see WNT at the kernel.
+template <int AUX = 0>
 __device__ __forceinline__ void dma16(const char* gptr, char* lds_wave_base) {
   __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(gptr),
-                                   (__attribute__((address_space(3))) uint32_t*)lds_wave_base, 16, 0, 0);
+                                   (__attribute__((address_space(3))) uint32_t*)lds_wave_base, 16, 0, AUX);
 }
 
 // Scheduling pattern: N_READS times (N_MFMA MFMAs, then one LDS read).
@@ -603,7 +606,13 @@ __device__ __forceinline__ void pair_reads() {
 // where every workgroup streams W rows of its own (one token tile), 2-3 % at 4096 x 1024 tokens x hidden, nothing from
 // 8192 x 4096 on; with the entropy or the argmax its fold spills and it only pays at one or two token tiles
 // (fused_plan holds the rule and the figures).
-template <bool ENT, bool AMAX, int NBT, int HI, bool DEEP = false>
+//
+// WNT: W is requested non-temporally.  Where W streams through once or a few times (up to four token tiles) its rows have
+// no business in the caches that the hidden rows and the partials live in: 64 x 4096 tokens x hidden 221 -> 205 us,
+// 256 x 1024 88 -> 84, 128 x 4096 234 -> 230, 512 x 1024 138 -> 135.5, 1024 x 4096 924 -> 917; from 2048 tokens on the
+// workgroups of an XCD that share a W tile want it kept (4096 x 1024: 936 -> 951), and so do three 128-token tiles
+// (384 x 1024: 130 -> 138).
+template <bool ENT, bool AMAX, int NBT, int HI, bool DEEP = false, bool WNT = false>
 __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   static_assert((NBT == 4 && (HI == 4 || HI == 3)) || (NBT != 4 && HI == 0), "256-token tile: every vocab tile 256 (HI = 4) or 224 rows; others: mixed heights");
@@ -748,7 +757,7 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
   // the code has no branch and the wait counts stay static.
   auto issue_piece = [&](int piece) {
     const unsigned slab = (unsigned)(issued < n_steps ? issued : n_steps - 1);
-    if (piece < k2Loads) dma16(pa[piece], smem + (slab % kBufsW) * kWBytes + wave * 1024 + piece * 8192);
+    if (piece < k2Loads) dma16<WNT ? 2 : 0>(pa[piece], smem + (slab % kBufsW) * kWBytes + wave * 1024 + piece * 8192);
     else dma16(pb[piece - k2Loads], smem + kHBase + (slab % kBufs) * kHBytes + wave * 1024 + (piece - k2Loads) * 8192);
   };
   auto issue_done = [&]() {
@@ -1311,6 +1320,7 @@ struct FusedPlan {
   int dma_nbt;                               // kDma only: token blocks per wave (4, 2 or 1: 256, 128 or 64 tokens per tile)
   int unit32;                                // kDma only: 32-row blocks per vocab unit (1 = mixed tile heights; 7 / 8 = whole tiles of 224 / 256 rows)
   int dma_deep;                              // kDma, 256-token tile only: three W buffers - 0 never, 1 for sweeps without the entropy, 2 always
+  bool w_nt;                                 // kDma only: W requested non-temporally (few token tiles: see the kernel's WNT)
   int small_nbt, small_ksteps, small_waves;  // kSmall only
   int bt, slots;
   int n_vunits, upt;   // vocab units the splits share out, and units per 256-row tile (what a unit costs, for the schedule)
@@ -1393,6 +1403,7 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   // registers around every tile change: 1024 x 4096 -3 %, but 4096 x 1024 +2.6 % and 8192 x 4096 +2.3 %.
   p.dma_deep = 0;
   if (p.dma_nbt == 4) p.dma_deep = n_tokens <= 1024 ? 2 : ((H < 4096 || n_tokens <= 8192) ? 1 : 0);
+  p.w_nt = p.dma_nbt == 4 ? n_tokens <= 1024 : n_tokens <= dma_tile_tokens(p.dma_nbt);
   p.unit32 = 8;   // 32-row blocks per vocab unit: whole 256-row tiles unless the DMA kernel is given something finer below
   if (H % k2BK == 0) p.kind = kDma;
   // The streaming kernel runs one workgroup per CU: without a CU count (no device) the tiled kernels serve.
@@ -1476,11 +1487,11 @@ size_t fused_workspace_bytes(int64_t n_tokens, int64_t H, int64_t V, int n_weigh
   return off_partials(n_tokens) + (size_t)n_weights * partial_bytes(n_tokens, H, V) + normed_bytes(n_tokens, H, with_norm);
 }
 
-template <bool ENT, bool AMAX, int NBT, int HI, bool DEEP = false>
+template <bool ENT, bool AMAX, int NBT, int HI, bool DEEP = false, bool WNT = false>
 static void launch_dma_nbt(const FusedArgs& a, int grid, hipStream_t stream) {
   static DeviceOnce attr_set;  // opt in to > 64 KB of dynamic LDS once per instantiation and device
   if (attr_set.first_on_current_device() &&
-      !allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI, DEEP>, dma_lds_bytes(NBT, DEEP)) && DEEP) {
+      !allow_big_lds(&fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI, DEEP, WNT>, dma_lds_bytes(NBT, DEEP)) && DEEP) {
     int dev = 0;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDeviceOrdinals)
       g_no_deep_lds.fetch_or(1ull << dev, std::memory_order_relaxed);
@@ -1488,17 +1499,22 @@ static void launch_dma_nbt(const FusedArgs& a, int grid, hipStream_t stream) {
   if constexpr (DEEP) {
     if (deep_lds_refused()) return launch_dma_nbt<ENT, AMAX, NBT, HI, false>(a, grid, stream);
   }
-  hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI, DEEP>), dim3((unsigned)grid), dim3(k2WG), dma_lds_bytes(NBT, DEEP),
-                     stream, a);
+  hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI, DEEP, WNT>), dim3((unsigned)grid), dim3(k2WG),
+                     dma_lds_bytes(NBT, DEEP), stream, a);
 }
+// w_nt: non-temporal W requests (the kernel's WNT; the 64-token tile always has them, its launches have one token tile).
 template <bool ENT, bool AMAX>
-static void launch_dma(const FusedArgs& a, int nbt, int unit32, bool deep, int grid, hipStream_t stream) {
-  if (nbt == 4 && unit32 == 7 && deep) launch_dma_nbt<ENT, AMAX, 4, 3, true>(a, grid, stream);
+static void launch_dma(const FusedArgs& a, int nbt, int unit32, bool deep, bool w_nt, int grid, hipStream_t stream) {
+  if (nbt == 4 && deep && w_nt) {
+    if (unit32 == 7) launch_dma_nbt<ENT, AMAX, 4, 3, true, true>(a, grid, stream);
+    else launch_dma_nbt<ENT, AMAX, 4, 4, true, true>(a, grid, stream);
+  } else if (nbt == 4 && unit32 == 7 && deep) launch_dma_nbt<ENT, AMAX, 4, 3, true>(a, grid, stream);
   else if (nbt == 4 && deep) launch_dma_nbt<ENT, AMAX, 4, 4, true>(a, grid, stream);
   else if (nbt == 4 && unit32 == 7) launch_dma_nbt<ENT, AMAX, 4, 3>(a, grid, stream);   // 224-row tiles
   else if (nbt == 4) launch_dma_nbt<ENT, AMAX, 4, 4>(a, grid, stream);
+  else if (nbt == 2 && w_nt) launch_dma_nbt<ENT, AMAX, 2, 0, false, true>(a, grid, stream);
   else if (nbt == 2) launch_dma_nbt<ENT, AMAX, 2, 0>(a, grid, stream);
-  else launch_dma_nbt<ENT, AMAX, 1, 0>(a, grid, stream);
+  else launch_dma_nbt<ENT, AMAX, 1, 0, false, true>(a, grid, stream);
 }
 
 template <bool ENT, bool AMAX, int NBT, int KSTEPS>
@@ -1534,8 +1550,8 @@ static int launch_main(const FusedArgs& a, const FusedPlan& plan, bool want_argm
     return n;  // >= 2: fused_plan only picks this kernel when it can be placed
   }
   if (plan.kind == kDma) {
-    if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.unit32, plan.dma_deep >= (ENT ? 2 : 1), plan.grid, stream);
-    else launch_dma<ENT, false>(a, plan.dma_nbt, plan.unit32, plan.dma_deep >= (ENT ? 2 : 1), plan.grid, stream);
+    if (want_argmax) launch_dma<ENT, true>(a, plan.dma_nbt, plan.unit32, plan.dma_deep >= (ENT ? 2 : 1), plan.w_nt, plan.grid, stream);
+    else launch_dma<ENT, false>(a, plan.dma_nbt, plan.unit32, plan.dma_deep >= (ENT ? 2 : 1), plan.w_nt, plan.grid, stream);
   } else {
     if (want_argmax) hipLaunchKernelGGL((fused_lmhead_kernel<ENT, true>), dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
     else hipLaunchKernelGGL((fused_lmhead_kernel<ENT, false>), dim3((unsigned)plan.grid), dim3(kFusedWG), 0, stream, a);
