@@ -1062,12 +1062,23 @@ def main():
         done("grpo_pair")
     if "small" in only:
         t = bench_fused(dev, K, W, n=64)
+        # the streaming kernel's own shapes: up to 16 tokens at H = 1024, up to 64 at larger hidden sizes
+        stream = {}
+        for n, H in ((16, 1024), (64, 2048)):
+            u = bench_fused(dev, K, W, n=n, H=H, seed=2000 + n + H)
+            stream[f"{n}x{H}"] = {**timing_fields(u),
+                                  "roofline": hbm_roofline(u["bytes"], u["ms"], None, "fused_lmhead_small_kernel + fused_combine_kernel")}
+            log(f"streaming kernel {n}x{H}: {u['ms'] * 1e3:.1f} us, {stream[f'{n}x{H}']['roofline']['frac']:.3f} of HBM peak")
+            torch.cuda.empty_cache()
         legs["fused_lmhead_decode_batch"] = {
             "value": t["tokens"] / (t["ms"] * 1e-3), "unit": "token-logprobs/s", **timing_fields(t),
             "dtype": "bf16 x bf16 -> f32",
-            "config": {"workload": "fused lm_head + log-softmax at a decode-step batch: hidden [64,1024] x W [151936,1024] bf16",
-                       "tokens": t["tokens"], "hidden": t["H"], "vocab": V},
-            "roofline": hbm_roofline(t["bytes"], t["ms"], traffic_of("fused_lmhead_small_64tokens"), "fused_lmhead_small_kernel")}
+            "config": {"workload": "fused lm_head + log-softmax at a decode-step batch: hidden [64,1024] x W [151936,1024] bf16 "
+                                   "(the tiled kernel's 64-token tile, W requested non-temporally); `streaming_kernel_shapes`: the "
+                                   "kernel that splits K over the waves, on shapes it serves",
+                       "tokens": t["tokens"], "hidden": t["H"], "vocab": V, "streaming_kernel_shapes": stream},
+            "roofline": hbm_roofline(t["bytes"], t["ms"], traffic_of("fused_lmhead_decode_64tokens"),
+                                     "fused_lmhead_dma_kernel<64-token tile> + fused_combine_kernel")}
         done("fused_lmhead_decode_batch")
     if "midsize" in only:   # batches of up to one token tile: W streams once, HBM-bound
         mid = {}

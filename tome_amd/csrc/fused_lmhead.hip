@@ -961,15 +961,14 @@ __global__ __launch_bounds__(k2WG) void fused_lmhead_dma_kernel(FusedArgs a) {
 //   * Per tile the waves' partial sums (16 rows x 16*NBT tokens, MFMA layout) meet in LDS; wave j sums
 //     them in wave order and folds token block j into its online-softmax state.  One barrier per tile:
 //     the buffer of tile t is rewritten at tile t + 2, after the barrier of tile t + 1, which the
-//     folding waves only reach once tile t is folded.  (Eight token blocks - 65..128 tokens, K slices of
-//     128 on 8 waves, H = 1024 only - use one buffer and a second barrier: two would not fit the LDS.)
+//     folding waves only reach once tile t is folded.
 //   * One partial per (token, workgroup); the combine kernel is shared with the other paths.
 // ===============================================================================================
 template <bool ENT, bool AMAX, int NBT, int KSTEPS>
 __global__ __launch_bounds__(512) void fused_lmhead_small_kernel(FusedArgs a) {
   extern __shared__ __attribute__((aligned(16))) char small_mem[];  // [2][waves][NBT][64 lanes] f32x4, then [waves] 4 KB tiles
-  constexpr int kBuf = NBT == 8 ? 2 : 16 / KSTEPS;                  // tile buffers in flight (registers): 16 loads, 8 with 8 token blocks
-  constexpr int kRed = NBT == 8 ? 1 : 2;                            // reduction buffers (LDS)
+  constexpr int kBuf = 16 / KSTEPS;                                 // tile buffers in flight (registers): 16 loads per lane
+  constexpr int kRed = 2;                                           // reduction buffers (LDS)
   const int n_valid = a.n_valid ? *a.n_valid : a.n_tokens;
   if (n_valid <= 0) return;
   const int lane = threadIdx.x & 63;
@@ -1075,7 +1074,6 @@ __global__ __launch_bounds__(512) void fused_lmhead_small_kernel(FusedArgs a) {
         for (int w = 0; w < n_waves; ++w) sum[0][0] += *reinterpret_cast<const f32x4v*>(src + (size_t)w * NBT * 1024);
         fold_tile16<ENT, AMAX, 1>(sum, st, tx, tgt, t * 16, g, t * 16 + 16 > a.V, a.V, a.scale);
       }
-      if constexpr (kRed == 1) __syncthreads();  // one buffer: the next tile's sums wait for this fold
     }
   }
   // One partial per (token, workgroup): part index = workgroup id.
@@ -1364,15 +1362,14 @@ static int small_wg_count() {
 }
 
 // Shape rules of the small-batch kernel: <= 64 tokens, K split over 2..8 waves in slices of 256 or 512
-// (slices of 128 on twice the waves measured 2 us slower at H = 1024); 65..128 tokens at H = 1024 only.
+// (slices of 128 on twice the waves measured 2 us slower at H = 1024).  At H = 1024 it keeps up to 16 tokens only: since
+// the tiled kernel requests W non-temporally where it streams through once, its 64- and 128-token tiles are faster there
+// from 17 tokens on (17..64 tokens: 53.3-54.8 against 54.7-59 us; 65..128, which this kernel served with eight token blocks
+// on K slices of 128: 61-64 against 67-72 us); at 1280, 1536 and 1792 the two are within 3 % of each other either way, at
+// 2048 and above this kernel wins (64 x 2048: 108 against 125 us).
 static bool small_shape(int64_t n_tokens, int64_t H, int64_t V, int& nbt, int& ksteps, int& waves) {
-  if (n_tokens > 128 || V < 64) return false;
-  if (n_tokens > 64) {  // eight token blocks: the B fragments only fit with K slices of 128, on exactly 8 waves
-    nbt = 8;
-    ksteps = 4;
-    waves = 8;
-    return H == 1024;
-  }
+  if (n_tokens > 64 || V < 64) return false;
+  if (H == 1024 && n_tokens > 16) return false;
   nbt = n_tokens <= 16 ? 1 : (n_tokens <= 32 ? 2 : 4);
   if (H % 256 == 0 && H / 256 <= 8 && H / 256 >= 2) {
     ksteps = 8;
@@ -1383,7 +1380,7 @@ static bool small_shape(int64_t n_tokens, int64_t H, int64_t V, int& nbt, int& k
   } else {
     return false;
   }
-  if (ksteps == 8 && nbt == 2) nbt = 4;  // instantiated token-block counts: 1 and 4 (K 256), 1 and 2 (K 512), 8 (K 128)
+  if (ksteps == 8 && nbt == 2) nbt = 4;  // instantiated token-block counts: 1 and 4 (K 256), 1 and 2 (K 512)
   return waves >= nbt;
 }
 
@@ -1415,12 +1412,12 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   if (forced == kForceDmaThreeWBuffers && p.dma_nbt == 4) p.dma_deep = 2;
   if (p.kind == kSmall) {
     // One partial per (token, workgroup); one workgroup per CU, at most 512.
-    p.bt = 128;
+    p.bt = 64;
     p.slots = 1;     // only feed the schedule that the compaction kernel writes and this path ignores
     p.n_vunits = 1;
     p.upt = 1;
     p.grid = 0;
-    p.max_records = (size_t)128 * 512;
+    p.max_records = (size_t)64 * 512;
     return p;
   }
   p.bt = p.kind == kGeneric ? kBT : dma_tile_tokens(p.dma_nbt);   // the DMA path: 256 vocab rows x 256, 128 or 64 tokens
@@ -1523,7 +1520,7 @@ static int launch_small(const FusedArgs& a, int waves, hipStream_t stream) {
   const int n_tiles = (a.V + 15) / 16;
   if (n_wg > n_tiles) n_wg = n_tiles & ~1;  // no empty vocab ranges
   if (n_wg < 2) return 0;
-  const size_t lds = (size_t)(NBT == 8 ? 1 : 2) * waves * NBT * 1024 + (size_t)waves * 4096;
+  const size_t lds = (size_t)2 * waves * NBT * 1024 + (size_t)waves * 4096;
   static DeviceOnce attr_set;  // opt in to > 64 KB of dynamic LDS once per instantiation and device
   if (lds > 65536 && attr_set.first_on_current_device())
     allow_big_lds(&fused_lmhead_small_kernel<ENT, AMAX, NBT, KSTEPS>, 2 * 8 * 4 * 1024 + 8 * 4096);
@@ -1541,8 +1538,7 @@ static int launch_main(const FusedArgs& a, const FusedPlan& plan, bool want_argm
     const int w = plan.small_waves;
 #define TOME_SMALL(NBT, KS)                                                 \
   n = want_argmax ? launch_small<ENT, true, NBT, KS>(a, w, stream) : launch_small<ENT, false, NBT, KS>(a, w, stream)
-    if (plan.small_nbt == 8) TOME_SMALL(8, 4);
-    else if (plan.small_ksteps == 8 && plan.small_nbt == 1) TOME_SMALL(1, 8);
+    if (plan.small_ksteps == 8 && plan.small_nbt == 1) TOME_SMALL(1, 8);
     else if (plan.small_ksteps == 8) TOME_SMALL(4, 8);
     else if (plan.small_nbt == 1) TOME_SMALL(1, 16);
     else TOME_SMALL(2, 16);
