@@ -358,8 +358,9 @@ def test_norm_lmhead_matches_oracle(dev, n, H, V, masked):
     (20, 2560, 9000, False), (5, 512, 7000, False), (64, 1536, 5000, False), (48, 1024, 70, False),
     (65, 1024, 5001, False), (100, 1024, 30000, True), (128, 1024, 151936, False), (128, 1024, 200, True)])
 def test_fused_small_batch_kernel(dev, n, H, V, masked):
-    """Decode-sized batches (<= 64 tokens; <= 128 at H = 1024) take the streaming kernel with K split across waves
-    (where the shape rules allow it; the other shapes here fall back to the tiled kernel) - same bar either way."""
+    """Decode-sized batches (<= 64 tokens; <= 16 at H = 1024) take the streaming kernel with K split across waves
+    (where the shape rules allow it; the other shapes here go to the tiled kernel's 64- and 128-token tiles, which
+    request W non-temporally) - same bar either way."""
     rng = np.random.default_rng(n * 31 + H + V)
     h, w, t = _inputs(dev, n, H, V, n * 31 + H + V, w_scale=0.05)
     valid = (rng.random(n) < 0.7).astype(np.int32) if masked else np.ones(n, dtype=np.int32)
@@ -380,7 +381,7 @@ def test_fused_small_batch_kernel(dev, n, H, V, masked):
 
 @pytest.mark.parametrize("n,H", [(10, 1024), (100, 1024), (50, 4096), (100, 2560), (300, 1024), (40, 72)])
 def test_fused_all_masked_and_single_valid_row(dev, n, H):
-    """Every sweep kernel (streaming with 1 / 4 / 8 token blocks, DMA with 64- / 128- / 256-token tiles, generic) with
+    """Every sweep kernel (streaming with 1 / 2 token blocks, DMA with 64- / 128- / 256-token tiles, generic) with
     no valid row at all - nothing may be read, every output is the masked value - and with exactly one."""
     V = 5000
     h, w, t = _inputs(dev, n, H, V, n + H, w_scale=0.05)
