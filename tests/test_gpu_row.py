@@ -280,6 +280,40 @@ def test_full_log_softmax_bf16_one_pass_and_its_limits(dev, rows, V, T):
     assert torch.equal(out2.view(torch.int16), out.view(torch.int16))
 
 
+@pytest.mark.parametrize("rows,V,pad,T", [(50, 20003, 5, 1.0), (64, 151941, 3, 0.7), (45, 16391, 9, 1.3)])
+def test_full_log_softmax_one_pass_with_single_trailing_elements(dev, rows, V, pad, T):
+    """Through the C ABI with padded row strides (a multiple of 8 elements, which the tensor wrapper's contiguous output
+    never has when V is not): the one-pass kernel then also takes rows whose last V % 8 elements are single elements.
+    Same bar as the other bf16 cases; the padding of the output rows stays untouched."""
+    from tome_amd import _lib
+    lib = tome_amd.load_library()
+    rng = np.random.default_rng(rows + V)
+    stride = V + pad
+    assert stride % 8 == 0
+    x32 = (rng.standard_normal((rows, V)) * 2).astype(np.float32)
+    x32[1, rng.random(V) < 0.3] = -np.inf
+    xin = torch.zeros((rows, stride), dtype=torch.bfloat16, device=dev)
+    xin[:, :V] = torch.from_numpy(x32).to(dev).to(torch.bfloat16)
+    out = torch.full((rows, stride), 7.0, dtype=torch.bfloat16, device=dev)
+    lse = torch.empty(rows, dtype=torch.float32, device=dev)
+    ws_bytes = lib.tome_row_logprob_workspace(rows, V)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    _lib.check(lib.tome_full_log_softmax(xin.data_ptr(), out.data_ptr(), 1, rows, V, stride, stride, T, lse.data_ptr(),
+                                         ws.data_ptr(), ws_bytes, torch.cuda.current_stream(dev).cuda_stream))
+    torch.cuda.synchronize()
+    bits = bf16_bits_of(xin[:, :V].contiguous())
+    want = oracle.fused_log_softmax_f32(bits, T)
+    got = bf16_bits_of(out[:, :V].contiguous())
+    a, b = oracle.bf16_to_f32(got), oracle.bf16_to_f32(want)
+    fin = np.isfinite(b)
+    np.testing.assert_array_equal(np.isneginf(a), np.isneginf(b))
+    diff = np.abs(a[fin] - b[fin])
+    assert (diff <= 0.125 + 1e-6).all() and (diff == 0).mean() > 0.99
+    assert (diff[-1000:] == 0).mean() > 0.98                                   # the trailing elements among them
+    np.testing.assert_allclose(lse.cpu().numpy(), oracle.lse_rows(bits, T), atol=2e-5 * max(1.0, 1.0 / T), rtol=1e-6)
+    assert (out[:, V:] == 7.0).all()
+
+
 def test_full_log_softmax_fp32_split_rows_merge_inside_the_second_pass(dev):
     """fp32 batches of fewer than 512 rows are split over several workgroups in the first pass; the second pass merges
     the partials itself.  Against the fp64 oracle at 1e-4, and the lse it leaves must equal token_logprobs' lse."""
