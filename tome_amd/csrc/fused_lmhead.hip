@@ -1400,7 +1400,10 @@ static FusedPlan fused_plan(int64_t n_tokens, int64_t H, int64_t V) {
   // registers around every tile change: 1024 x 4096 -3 %, but 4096 x 1024 +2.6 % and 8192 x 4096 +2.3 %.
   p.dma_deep = 0;
   if (p.dma_nbt == 4) p.dma_deep = n_tokens <= 1024 ? 2 : ((H < 4096 || n_tokens <= 8192) ? 1 : 0);
-  p.w_nt = p.dma_nbt == 4 ? n_tokens <= 1024 : n_tokens <= dma_tile_tokens(p.dma_nbt);
+  // Non-temporal W (the kernel's WNT): few token tiles, and a W larger than the 256 MB memory-side cache - a smaller one is
+  // found there again by the next call as long as it is requested normally (repeated calls, 64 tokens: V = 32000, H = 4096,
+  // 262 MB: 48 us against 71 non-temporally; V = 50257, H = 768, 77 MB: 21.0 against 23.3).
+  p.w_nt = (p.dma_nbt == 4 ? n_tokens <= 1024 : n_tokens <= dma_tile_tokens(p.dma_nbt)) && V * H * 2 >= (int64_t)288 << 20;
   p.unit32 = 8;   // 32-row blocks per vocab unit: whole 256-row tiles unless the DMA kernel is given something finer below
   if (H % k2BK == 0) p.kind = kDma;
   // The streaming kernel runs one workgroup per CU: without a CU count (no device) the tiled kernels serve.
@@ -1499,7 +1502,7 @@ static void launch_dma_nbt(const FusedArgs& a, int grid, hipStream_t stream) {
   hipLaunchKernelGGL((fused_lmhead_dma_kernel<ENT, AMAX, NBT, HI, DEEP, WNT>), dim3((unsigned)grid), dim3(k2WG),
                      dma_lds_bytes(NBT, DEEP), stream, a);
 }
-// w_nt: non-temporal W requests (the kernel's WNT; the 64-token tile always has them, its launches have one token tile).
+// w_nt: non-temporal W requests (the kernel's WNT).
 template <bool ENT, bool AMAX>
 static void launch_dma(const FusedArgs& a, int nbt, int unit32, bool deep, bool w_nt, int grid, hipStream_t stream) {
   if (nbt == 4 && deep && w_nt) {
@@ -1511,7 +1514,8 @@ static void launch_dma(const FusedArgs& a, int nbt, int unit32, bool deep, bool 
   else if (nbt == 4) launch_dma_nbt<ENT, AMAX, 4, 4>(a, grid, stream);
   else if (nbt == 2 && w_nt) launch_dma_nbt<ENT, AMAX, 2, 0, false, true>(a, grid, stream);
   else if (nbt == 2) launch_dma_nbt<ENT, AMAX, 2, 0>(a, grid, stream);
-  else launch_dma_nbt<ENT, AMAX, 1, 0, false, true>(a, grid, stream);
+  else if (w_nt) launch_dma_nbt<ENT, AMAX, 1, 0, false, true>(a, grid, stream);
+  else launch_dma_nbt<ENT, AMAX, 1, 0>(a, grid, stream);
 }
 
 template <bool ENT, bool AMAX, int NBT, int KSTEPS>
