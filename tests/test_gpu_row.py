@@ -147,9 +147,8 @@ def test_local_compute_logprobs_dropin(dev):
 @pytest.mark.parametrize("rows,V,T", [(1, V_QWEN3, 1.0), (3, 4096 * 2 + 1, 0.7), (64, 4096, 1.0), (5, 8192 + 384, 2.0),
                                       (1400, 4100, 1.0), (1301, 1030, 0.7), (40, 2051, 1.3)])
 def test_fused_log_softmax_full_matrix(dev, dtype, rows, V, T):
-    """model.py:77-89 drop-in, incl. the kernel's tail cases (V % 4096 in {0, 1, 384}) and, for fp32, both sizes of the
-    second pass's workgroups (two loads per lane below 1300 rows, one from there on) with rows that end in a partial
-    workgroup and in single elements."""
+    """model.py:77-89 drop-in, incl. the kernel's tail cases (V % 4096 in {0, 1, 384}) and batches of more rows than
+    workgroups fit the chip at once, with rows that end in a partial workgroup and in single elements."""
     rng = np.random.default_rng(V + rows)
     x = torch.from_numpy(rng.standard_normal((rows, V)).astype(np.float32)).to(dev).to(dtype)
     out = tome_amd.fused_log_softmax(x, T)
@@ -312,6 +311,25 @@ def test_full_log_softmax_one_pass_with_single_trailing_elements(dev, rows, V, p
     assert (diff[-1000:] == 0).mean() > 0.98                                   # the trailing elements among them
     np.testing.assert_allclose(lse.cpu().numpy(), oracle.lse_rows(bits, T), atol=2e-5 * max(1.0, 1.0 / T), rtol=1e-6)
     assert (out[:, V:] == 7.0).all()
+
+
+def test_full_log_softmax_fp32_above_three_quarters_of_a_gigabyte(dev):
+    """fp32 matrices above 3/4 GB: the first pass streams the rows past the caches and the second pass runs workgroups of one
+    load per lane.  Too large for the fp64 oracle as a whole: 24 rows spread over the matrix against it at 1e-4, every row's
+    probabilities summing to one, and the last elements of the last row (a ragged V) in place."""
+    rows, V, T = 1400, V_QWEN3 + 3, 0.9
+    g = torch.Generator(device=dev).manual_seed(9)
+    x = torch.empty((rows, V), dtype=torch.float32, device=dev)
+    for i in range(0, rows, 200):
+        x[i:i + 200] = torch.randn((min(200, rows - i), V), device=dev, generator=g) * 2
+    out = tome_amd.fused_log_softmax(x, T)
+    pick = np.linspace(0, rows - 1, 24).astype(np.int64)
+    want = oracle.full_log_softmax64(x[torch.from_numpy(pick).to(dev)].cpu().numpy(), T)
+    np.testing.assert_allclose(out[torch.from_numpy(pick).to(dev)].cpu().numpy(), want, atol=TOL_F32, rtol=0)
+    total = torch.exp(out.double()).sum(-1)
+    assert (total - 1.0).abs().max().item() < 1e-4
+    del out, x
+    torch.cuda.empty_cache()
 
 
 def test_full_log_softmax_fp32_split_rows_merge_inside_the_second_pass(dev):

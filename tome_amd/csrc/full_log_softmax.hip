@@ -284,11 +284,13 @@ hipError_t full_log_softmax_launch(const void* in, void* out, int dtype, int64_t
   // Many short workgroups stream a read + write mix best, as long as each still issues a few loads per lane.  bf16
   // rows (a batch too small or rows too long for the one-pass kernel): four loads per lane and pass, aiming at 65536
   // workgroups (against 4096: 4096 x 151936 bf16 655 -> 633 us, both passes included).  fp32 rows: workgroups of ONE pass
-  // of two loads per lane - of one load per lane from ~1300 rows on (both passes, rows of 151936 fp32, four / two / one load:
-  // 64 rows 24.4 / 24.2 / 26.6 us, 1024 rows 296 / 288 / 295, 2048 rows 629 / 618 / 588, 4096 rows 1370 / 1227 / 1168).
+  // of two loads per lane - of one load per lane for matrices above 3/4 GB, the size up to which the first pass leaves the
+  // rows in the caches (both passes, rows of 151936 fp32, four / two / one load: 64 rows 24.4 / 24.2 / 26.6 us, 1024 rows
+  // 296 / 288 / 295, 2048 rows 629 / 618 / 588, 4096 rows 1370 / 1227 / 1168; rows of 32000: 4096 rows - / 248 / 253,
+  // 8192 rows - / 503 / 491; rows of 65536: 2048 rows - / 254 / 256, 4096 rows - / 501 / 496).
   int64_t chunks = (65536 + rows - 1) / rows;
   int64_t by_work = units / (kFullUnroll * kFullWG);
-  const int f32_unroll = rows >= 1300 ? 1 : 2;
+  const int f32_unroll = (double)rows * (double)V * 4.0 > 768.0 * 1024 * 1024 ? 1 : 2;
   if (dtype == 0 && vector_ok) {
     chunks = by_work = units / (f32_unroll * kFullWG);
   }
