@@ -150,9 +150,10 @@ int tome_row_sample(const void* logits, int dtype, int64_t rows, int64_t V, int6
  * (mlx-impl/model.py:77-89): out[r, j] = T(x[r, j] * (1/temp)) - T(lse_r), same shape
  * and dtype as the input, the subtraction carried out in the I/O dtype (model.py:57,60).
  * `row_lse` is a caller-provided float32 buffer of `rows` elements (it receives the rows' lse);
- * workspace: tome_row_logprob_workspace(rows, V).  Batches of 44 and more bf16 rows of 16384 .. 155648
- * elements with 16-byte aligned rows are read once and written once (the row stays in one workgroup's registers);
- * everything else is read twice and written once, where the reference reads three times.
+ * workspace: tome_row_logprob_workspace(rows, V).  bf16 rows of 16384 .. 155648 elements with 16-byte aligned
+ * rows are read once and written once (the row stays in one workgroup's registers), except for batches of a few dozen
+ * rows or fewer when the rows are longer than 40960 elements; everything else is read twice and written once, where the
+ * reference reads three times.
  */
 int tome_full_log_softmax(const void* logits, void* out, int dtype, int64_t rows, int64_t V,
                           int64_t in_row_stride, int64_t out_row_stride, float temperature,

@@ -232,13 +232,17 @@ constexpr int kOnePassUnits = 19;  // 16-byte units per lane: 1024 lanes hold 15
 
 // Whether the one-pass kernel takes this call: bf16, 16-byte aligned rows, a row that fits the registers of one
 // workgroup and is long enough to keep most of its 1024 lanes busy.
-// One workgroup per row leaves most of the chip idle on a decode-sized batch: below ~44 rows the two-pass kernels, which
-// split a row over several workgroups, are faster (8 / 32 / 48 / 64 / 80 rows of 151936 bf16: 8.1 / 11.6 / 14.3 / 16.5 /
-// 19.4 us against 12.8 / 13.2 / 13.3 / 13.4 / 13.7; 128 / 512 / 2048 rows: 25.4 / 77.5 / 291 against 16.9 / 58.4 / 227).
+// One workgroup per row leaves most of the chip idle on a decode-sized batch, but it is ONE launch where the two-pass form
+// is two: rows of up to 40960 elements always come here (16 rows of 16384 / 32000: 4.3 / 5.4 us against 6.8 / 7.9), longer
+// ones from V / 3000 rows on.  Measured crossovers: 65536 elements ~24 rows (16 rows 7.5 against 7.0 us, 32 rows 7.5
+// against 8.0), 131072 ~60 rows (32 rows 12.1 against 8.7, 64 rows 12.4 against 12.8), 151936 ~44 rows (32 / 48 / 64 rows:
+// 13.2 / 13.3 / 13.4 against 11.6 / 14.3 / 16.5); larger batches of 151936: 128 / 512 / 2048 rows 16.9 / 58.4 / 227 against
+// 25.4 / 77.5 / 291.
 bool full_log_softmax_one_pass(const void* in, const void* out, int dtype, int64_t rows, int64_t V, int64_t in_stride, int64_t out_stride) {
   const bool aligned = reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
                        in_stride % 8 == 0 && out_stride % 8 == 0;
-  return dtype == 1 && aligned && rows >= 44 && V >= 16384 && V / 8 <= (int64_t)kOnePassUnits * 1024;
+  const bool enough_rows = V <= 40960 || rows * 3000 >= V;
+  return dtype == 1 && aligned && enough_rows && V >= 16384 && V / 8 <= (int64_t)kOnePassUnits * 1024;
 }
 
 hipError_t full_log_softmax_onepass_launch(const void* in, void* out, int64_t rows, int64_t V, int64_t in_stride,
